@@ -38,7 +38,8 @@ def read_config_json(model_dir: str | Path) -> dict[str, Any]:
 
 
 def read_architecture(data: Mapping[str, Any]) -> str:
-    """The registry key of a configuration: ``architectures[0]``, else ``model_type``.
+    """The registry key of a configuration: ``architectures[0]``, else ``model_type``, else
+    ``architecture`` (a single name, as some model folders spell it).
 
     The reference keys its registry on ``model_type`` (rapid_llm/models/registry.py:44-78);
     both spellings are accepted here and resolved by the registry.
@@ -46,10 +47,11 @@ def read_architecture(data: Mapping[str, Any]) -> str:
     archs = data.get("architectures")
     if isinstance(archs, (list, tuple)) and archs and isinstance(archs[0], str):
         return archs[0]
-    model_type = data.get("model_type")
-    if isinstance(model_type, str) and model_type:
-        return model_type
-    raise ConfigError("config.json names neither 'architectures' nor 'model_type'")
+    for key in ("model_type", "architecture"):
+        name = data.get(key)
+        if isinstance(name, str) and name:
+            return name
+    raise ConfigError("config.json names neither 'architectures' nor 'model_type' nor 'architecture'")
 
 
 _DTYPE_NAMES = {

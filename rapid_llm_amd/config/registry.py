@@ -35,6 +35,8 @@ _ALIASES: dict[str, str] = {}
 _LAZY: dict[str, str] = {
     "Qwen3ForCausalLM": "rapid_llm_amd.models.qwen3",
     "qwen3": "rapid_llm_amd.models.qwen3",
+    "Fokulorn": "rapid_llm_amd.models.fokulorn",
+    "fokulorn": "rapid_llm_amd.models.fokulorn",
 }
 
 

@@ -4,7 +4,7 @@
 #include "common.h"
 
 // --------------------------------------------------------------------------- //
-// embedding: residual[t, :] = table[ids[t], :]   (float32 residual stream)
+// embedding: residual[t, :] = table[ids[t], :] * scale   (float32 residual stream)
 // rapid_llm/modules/vocab_parallel.py:102-103
 // --------------------------------------------------------------------------- //
 // A negative id -(r + 1) stands for "the token chosen in row r of the previous step", which
@@ -13,7 +13,7 @@
 template <typename W>
 __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ fed, int fed_rows,
                              const W* __restrict__ table, float* __restrict__ out, int hidden,
-                             int vocab) {
+                             int vocab, float scale) {
     const int t = blockIdx.x;
     int id = ids[t];
     if (id < 0 && fed && -id - 1 < fed_rows) id = fed[-id - 1];
@@ -30,25 +30,26 @@ __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict_
             const Pack p = *reinterpret_cast<const Pack*>(row + i);
 #pragma unroll
             for (int j = 0; j < VEC; j += 4)
-                *reinterpret_cast<float4*>(dst + i + j) = make_float4(
-                    to_float(p.v[j]), to_float(p.v[j + 1]), to_float(p.v[j + 2]), to_float(p.v[j + 3]));
+                *reinterpret_cast<float4*>(dst + i + j) =
+                    make_float4(to_float(p.v[j]) * scale, to_float(p.v[j + 1]) * scale,
+                                to_float(p.v[j + 2]) * scale, to_float(p.v[j + 3]) * scale);
         }
         return;
     }
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]) * scale;
 }
 
 extern "C" int rl_embed(const int* ids, const int* fed, int fed_rows, const void* table,
-                        int table_type, float* out, int tokens, int hidden, int vocab,
+                        int table_type, float* out, int tokens, int hidden, int vocab, float scale,
                         hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     dim3 grid(tokens), block(256);
     if (table_type == RL_F32)
         hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, fed, fed_rows,
-                           (const float*)table, out, hidden, vocab);
+                           (const float*)table, out, hidden, vocab, scale);
     else if (table_type == RL_BF16)
         hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, fed, fed_rows,
-                           (const bf16_t*)table, out, hidden, vocab);
+                           (const bf16_t*)table, out, hidden, vocab, scale);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -268,12 +269,23 @@ extern "C" int rl_add_rmsnorm_parts(float* residual, const float* parts, int npa
 }
 
 // --------------------------------------------------------------------------- //
-// SwiGLU on the packed [gate | up] row: out[:, j] = silu(x[:, j]) * x[:, I + j]
-// rapid_llm/kernels/ops/activation/swiglu.py:91-121
+// Gated activation on the packed [gate | up] row: out[:, j] = act(x[:, j], x[:, I + j]).
+// limit <= 0: SwiGLU, silu(g) * u (rapid_llm/kernels/ops/activation/swiglu.py:91-121).
+// limit > 0: the clamped variant, g' = min(g, limit), u' = clamp(u, -limit, limit),
+// g' * sigmoid(alpha * g') * (u' + 1).
 // --------------------------------------------------------------------------- //
+__device__ inline float glu_act(float g, float u, float limit, float alpha) {
+    if (limit > 0.f) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+    }
+    return g / (1.f + expf(-g)) * u;
+}
+
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter,
-                              size_t total) {
+                              size_t total, float limit, float alpha) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t step = (size_t)gridDim.x * blockDim.x;
     for (; idx < total; idx += step) {
@@ -282,8 +294,7 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
         const T* row = gate_up + t * 2 * (size_t)inter;
         const float g = to_float(row[j]);
         const float u = to_float(row[inter + j]);
-        const float s = g / (1.f + expf(-g));
-        out[idx] = from_float<T>(s * u);
+        out[idx] = from_float<T>(glu_act(g, u, limit, alpha));
     }
 }
 
@@ -295,7 +306,7 @@ struct alignas(sizeof(T) * 8) Vec8 {
 
 template <typename T>
 __global__ void swiglu_vec_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter,
-                                  size_t total_vec) {
+                                  size_t total_vec, float limit, float alpha) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t step = (size_t)gridDim.x * blockDim.x;
     const int per_row = inter >> 3;
@@ -308,37 +319,37 @@ __global__ void swiglu_vec_kernel(const T* __restrict__ gate_up, T* __restrict__
         Vec8<T> y;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const float gf = to_float(g.v[i]);
-            y.v[i] = from_float<T>(gf / (1.f + expf(-gf)) * to_float(u.v[i]));
+            y.v[i] = from_float<T>(glu_act(to_float(g.v[i]), to_float(u.v[i]), limit, alpha));
         }
         *reinterpret_cast<Vec8<T>*>(out + t * (size_t)inter + j) = y;
     }
 }
 
 template <typename T>
-static void launch_swiglu(const T* gate_up, T* out, int tokens, int inter, hipStream_t stream) {
+static void launch_swiglu(const T* gate_up, T* out, int tokens, int inter, float limit, float alpha,
+                          hipStream_t stream) {
     if (inter % 8 == 0) {
         const size_t total = (size_t)tokens * (inter / 8);
         size_t blocks = (total + 255) / 256;
         if (blocks > 65536) blocks = 65536;
         hipLaunchKernelGGL(swiglu_vec_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                           gate_up, out, inter, total);
+                           gate_up, out, inter, total, limit, alpha);
         return;
     }
     const size_t total = (size_t)tokens * inter;
     size_t blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     hipLaunchKernelGGL(swiglu_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, gate_up, out,
-                       inter, total);
+                       inter, total, limit, alpha);
 }
 
 extern "C" int rl_swiglu(const void* gate_up, void* out, int tokens, int inter, int act_type,
-                         hipStream_t stream) {
+                         float limit, float alpha, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (act_type == RL_F32)
-        launch_swiglu<float>((const float*)gate_up, (float*)out, tokens, inter, stream);
+        launch_swiglu<float>((const float*)gate_up, (float*)out, tokens, inter, limit, alpha, stream);
     else if (act_type == RL_BF16)
-        launch_swiglu<bf16_t>((const bf16_t*)gate_up, (bf16_t*)out, tokens, inter, stream);
+        launch_swiglu<bf16_t>((const bf16_t*)gate_up, (bf16_t*)out, tokens, inter, limit, alpha, stream);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -407,6 +418,43 @@ extern "C" int rl_add_bias(void* y, const float* bias, int rows, int cols, int a
 }
 
 // --------------------------------------------------------------------------- //
+// gate of a head: y[t, h, :] *= sigmoid(packed[t, gate_col + h]), one number a head, read
+// from a column of the row that the mixer's packed projection wrote
+// --------------------------------------------------------------------------- //
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ y, const T* __restrict__ packed, int row_width,
+                                 int gate_col, int heads, int d, size_t total) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    const size_t per_token = (size_t)heads * d;
+    for (; idx < total; idx += step) {
+        const size_t t = idx / per_token;
+        const int h = (int)((idx - t * per_token) / d);
+        const float g = to_float(packed[t * row_width + gate_col + h]);
+        y[idx] = from_float<T>(to_float(y[idx]) / (1.f + expf(-g)));
+    }
+}
+
+extern "C" int rl_head_gate(void* y, const void* packed, int row_width, int gate_col, int tokens,
+                            int heads, int d, int act_type, hipStream_t stream) {
+    if (tokens <= 0 || heads <= 0 || d <= 0) return RL_OK;
+    if (gate_col < 0 || gate_col + heads > row_width) return RL_ERR_ARG;
+    const size_t total = (size_t)tokens * heads * d;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    dim3 grid((unsigned)blocks), block(256);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(head_gate_kernel<float>, grid, block, 0, stream, (float*)y, (const float*)packed,
+                           row_width, gate_col, heads, d, total);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(head_gate_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, (const bf16_t*)packed,
+                           row_width, gate_col, heads, d, total);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
 // rotation tables: cos/sin[p, i] of the float32 product p * inv_freq[i]
 // rapid_llm/modules/rotary_embedding.py:194-202 (float32 outer product, then cos/sin)
 // --------------------------------------------------------------------------- //
@@ -465,7 +513,7 @@ __global__ void qknorm_rope_kvwrite_kernel(
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int d, int rotary_half, int interleaved, float eps,
-    int write_cache, int write_values, int head0) {
+    int write_cache, int write_values, int head0, int row_width, int v_head0) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -473,7 +521,7 @@ __global__ void qknorm_rope_kvwrite_kernel(
     const int half = d / 2;
     const int pos = positions[t];
     const int total_heads = nq + 2 * nkv;
-    const T* row = qkv + (size_t)t * total_heads * d;
+    const T* row = qkv + (size_t)t * row_width;
 
     size_t page = 0;
     int off = 0;
@@ -490,8 +538,9 @@ __global__ void qknorm_rope_kvwrite_kernel(
             // value head: copy into the transposed page (unless the tile kernel below does it)
             if (!write_cache || !write_values) continue;
             const int h = head - nq - nkv;
+            const T* xv = row + (size_t)(v_head0 + h) * d;  // where the row keeps this value head
             T* dst = v_cache + ((page * nkv + h) * d) * page_size + off;
-            for (int i = lane; i < d; i += RL_WAVE) dst[(size_t)i * page_size] = x[i];
+            for (int i = lane; i < d; i += RL_WAVE) dst[(size_t)i * page_size] = xv[i];
             continue;
         }
         const bool is_q = head < nq;
@@ -561,7 +610,8 @@ __device__ inline void qknorm_rope_kvwrite_vec(
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values, int head0) {
+    int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values, int head0,
+    int row_width, int v_head0) {
     constexpr int HPW = RL_WAVE / LPH;  // heads per wave
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -570,7 +620,7 @@ __device__ inline void qknorm_rope_kvwrite_vec(
     const int half = d / 2;
     const int pos = positions[t];
     const int total_heads = nq + (write_values ? 2 * nkv : nkv);
-    const T* row = qkv + (size_t)t * (nq + 2 * nkv) * d;
+    const T* row = qkv + (size_t)t * row_width;
     size_t page = 0;
     int off = 0;
     if (write_cache) {
@@ -584,8 +634,9 @@ __device__ inline void qknorm_rope_kvwrite_vec(
     if (head >= nq + nkv) {
         if (!write_cache) return;
         const int h = head - nq - nkv;
+        const T* xv = row + (size_t)(v_head0 + h) * d;
         T* dst = v_cache + ((page * nkv + h) * d) * page_size + off;
-        for (int i = li; i < d; i += LPH) dst[(size_t)i * page_size] = x[i];
+        for (int i = li; i < d; i += LPH) dst[(size_t)i * page_size] = xv[i];
         return;
     }
     const bool is_q = head < nq;
@@ -646,10 +697,12 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_vec_kernel(
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values, int head0) {
+    int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values, int head0,
+    int row_width, int v_head0) {
     qknorm_rope_kvwrite_vec<T, LPH>(blockIdx.x, blockIdx.y, qkv, q_out, k_cache, v_cache, q_norm_w, k_norm_w,
                                     cos_tab, sin_tab, positions, token_slot, block_table, table_stride,
-                                    page_size, nq, nkv, d, eps, write_cache, write_values, head0);
+                                    page_size, nq, nkv, d, eps, write_cache, write_values, head0, row_width,
+                                    v_head0);
 }
 
 template <typename T>
@@ -658,7 +711,7 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
                           const int* positions, const int* token_slot, const int* block_table,
                           int table_stride, int page_size, int tokens, int nq, int nkv, int d,
                           int rotary_half, int interleaved, float eps, int write_cache,
-                          int write_values, int head0, hipStream_t stream) {
+                          int write_values, int head0, int row_width, int v_head0, hipStream_t stream) {
     const int total_heads = nq + (write_values ? 2 * nkv : nkv) - head0;  // heads to work on
     // the vectorised kernel: head sizes in steps of 8, the half-split rotation of the whole head
     if (d % 8 == 0 && (!cos_tab || (rotary_half == d / 2 && !interleaved))) {
@@ -670,12 +723,12 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
             hipLaunchKernelGGL((qknorm_rope_kvwrite_vec_kernel<T, 16>), grid, block, 0, stream, qkv,
                                q_out, k_cache, v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab,
                                positions, token_slot, block_table, table_stride, page_size, nq, nkv,
-                               d, eps, write_cache, write_values, head0);
+                               d, eps, write_cache, write_values, head0, row_width, v_head0);
         else
             hipLaunchKernelGGL((qknorm_rope_kvwrite_vec_kernel<T, 32>), grid, block, 0, stream, qkv,
                                q_out, k_cache, v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab,
                                positions, token_slot, block_table, table_stride, page_size, nq, nkv,
-                               d, eps, write_cache, write_values, head0);
+                               d, eps, write_cache, write_values, head0, row_width, v_head0);
         return;
     }
     const int head_groups = (total_heads + 3) / 4;
@@ -683,7 +736,7 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
     hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<T>, grid, block, 0, stream, qkv, q_out, k_cache,
                        v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                        block_table, table_stride, page_size, nq, nkv, d, rotary_half, interleaved, eps,
-                       write_cache, write_values, head0);
+                       write_cache, write_values, head0, row_width, v_head0);
 }
 
 // Values of 16 consecutive tokens of the batch and one kv head, written by one workgroup.
@@ -699,12 +752,11 @@ template <typename T>
 __device__ inline void v_tile_write(
     int tile, int h, const T* __restrict__ qkv, T* __restrict__ v_cache, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int tokens, int nq, int nkv, int d) {
+    int page_size, int tokens, int nq, int nkv, int d, int row_width, int v_head0) {
     __shared__ T vt[VT_TOKENS][256 + 8];
     __shared__ int s_page[VT_TOKENS];
     __shared__ int s_off[VT_TOKENS];
     const int t0 = tile * VT_TOKENS;
-    const int row_width = (nq + 2 * nkv) * d;
     if (threadIdx.x < VT_TOKENS) {
         const int t = t0 + threadIdx.x;
         int page = -1, off = 0;
@@ -719,7 +771,7 @@ __device__ inline void v_tile_write(
     for (int idx = threadIdx.x; idx < VT_TOKENS * d; idx += 256) {
         const int i = idx / d, c = idx - i * d;
         if (t0 + i < tokens)
-            vt[i][c] = qkv[(size_t)(t0 + i) * row_width + (size_t)(nq + nkv + h) * d + c];
+            vt[i][c] = qkv[(size_t)(t0 + i) * row_width + (size_t)(v_head0 + h) * d + c];
     }
     __syncthreads();
     for (int idx = threadIdx.x; idx < 4 * d; idx += 256) {
@@ -756,16 +808,18 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int tokens, int head_groups, int nq, int nkv, int d, float eps, int head0) {
+    int page_size, int tokens, int head_groups, int nq, int nkv, int d, float eps, int head0,
+    int row_width, int v_head0) {
     const int qk_blocks = tokens * head_groups;
     if ((int)blockIdx.x < qk_blocks) {
         qknorm_rope_kvwrite_vec<T, LPH>(blockIdx.x / head_groups, blockIdx.x % head_groups, qkv, q_out, k_cache,
                                         v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
-                                        block_table, table_stride, page_size, nq, nkv, d, eps, 1, 0, head0);
+                                        block_table, table_stride, page_size, nq, nkv, d, eps, 1, 0, head0,
+                                        row_width, v_head0);
     } else {
         const int b = blockIdx.x - qk_blocks;
         v_tile_write<T>(b / nkv, b % nkv, qkv, v_cache, positions, token_slot, block_table, table_stride,
-                        page_size, tokens, nq, nkv, d);
+                        page_size, tokens, nq, nkv, d, row_width, v_head0);
     }
 }
 
@@ -773,9 +827,9 @@ template <typename T>
 __global__ __launch_bounds__(256) void v_tile_write_kernel(
     const T* __restrict__ qkv, T* __restrict__ v_cache, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int tokens, int nq, int nkv, int d) {
+    int page_size, int tokens, int nq, int nkv, int d, int row_width, int v_head0) {
     v_tile_write<T>(blockIdx.x, blockIdx.y, qkv, v_cache, positions, token_slot, block_table, table_stride,
-                    page_size, tokens, nq, nkv, d);
+                    page_size, tokens, nq, nkv, d, row_width, v_head0);
 }
 
 // true if it launched: head sizes in steps of 8, and a grid that fits
@@ -784,7 +838,7 @@ static bool launch_qkv_prepare(const T* qkv, T* q_out, T* k_cache, T* v_cache, c
                                const float* k_norm_w, const float* cos_tab, const float* sin_tab,
                                const int* positions, const int* token_slot, const int* block_table,
                                int table_stride, int page_size, int tokens, int nq, int nkv, int d,
-                               float eps, int head0, hipStream_t stream) {
+                               float eps, int head0, int row_width, int v_head0, hipStream_t stream) {
     if (d % 8) return false;
     const int lph = d <= 128 ? 16 : 32;
     const int heads_per_block = 4 * (RL_WAVE / lph);
@@ -795,11 +849,13 @@ static bool launch_qkv_prepare(const T* qkv, T* q_out, T* k_cache, T* v_cache, c
     if (lph == 16)
         hipLaunchKernelGGL((qkv_prepare_kernel<T, 16>), grid, block, 0, stream, qkv, q_out, k_cache, v_cache,
                            q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                           table_stride, page_size, tokens, head_groups, nq, nkv, d, eps, head0);
+                           table_stride, page_size, tokens, head_groups, nq, nkv, d, eps, head0, row_width,
+                           v_head0);
     else
         hipLaunchKernelGGL((qkv_prepare_kernel<T, 32>), grid, block, 0, stream, qkv, q_out, k_cache, v_cache,
                            q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                           table_stride, page_size, tokens, head_groups, nq, nkv, d, eps, head0);
+                           table_stride, page_size, tokens, head_groups, nq, nkv, d, eps, head0, row_width,
+                           v_head0);
     return true;
 }
 
@@ -809,10 +865,13 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
                                       const int* positions, const int* token_slot,
                                       const int* block_table, int table_stride, int page_size,
                                       int tokens, int nq, int nkv, int d, int rotary_half,
-                                      int interleaved, float eps, int write_cache, int act_type,
-                                      hipStream_t stream) {
+                                      int interleaved, float eps, int write_cache, int row_width,
+                                      int v_head0, int act_type, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (d % 2 || d > 256) return RL_ERR_ARG;
+    // the packed row: query heads from column 0, key heads behind them, the value heads from
+    // head v_head0 on (nq + nkv: behind the keys; nq: the values are the unrotated keys)
+    if (v_head0 < 0 || row_width < (nq + nkv) * d || (v_head0 + nkv) * d > row_width) return RL_ERR_ARG;
     // q_out null: the attention kernels finish the query heads themselves, and the work here
     // starts at the first key head
     const int head0 = q_out ? 0 : nq;
@@ -829,31 +888,34 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
     if (tile_values && whole_split && act_type == RL_F32 &&
         launch_qkv_prepare<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache, q_norm_w,
                                   k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                                  table_stride, page_size, tokens, nq, nkv, d, eps, head0, stream))
+                                  table_stride, page_size, tokens, nq, nkv, d, eps, head0, row_width, v_head0,
+                                  stream))
         return rl_launch_status();
     if (tile_values && whole_split && act_type == RL_BF16 &&
         launch_qkv_prepare<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                                    q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                                   table_stride, page_size, tokens, nq, nkv, d, eps, head0, stream))
+                                   table_stride, page_size, tokens, nq, nkv, d, eps, head0, row_width, v_head0,
+                                   stream))
         return rl_launch_status();
     if (act_type == RL_F32) {
         launch_qknorm<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache,
                              q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                              block_table, table_stride, page_size, tokens, nq, nkv, d, rotary_half,
-                             interleaved, eps, write_cache, !tile_values, head0, stream);
+                             interleaved, eps, write_cache, !tile_values, head0, row_width, v_head0, stream);
         if (tile_values)
             hipLaunchKernelGGL(v_tile_write_kernel<float>, vgrid, block, 0, stream,
                                (const float*)qkv, (float*)v_cache, positions, token_slot,
-                               block_table, table_stride, page_size, tokens, nq, nkv, d);
+                               block_table, table_stride, page_size, tokens, nq, nkv, d, row_width, v_head0);
     } else if (act_type == RL_BF16) {
         launch_qknorm<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
                               (bf16_t*)v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions,
                               token_slot, block_table, table_stride, page_size, tokens, nq, nkv, d,
-                              rotary_half, interleaved, eps, write_cache, !tile_values, head0, stream);
+                              rotary_half, interleaved, eps, write_cache, !tile_values, head0, row_width,
+                              v_head0, stream);
         if (tile_values)
             hipLaunchKernelGGL(v_tile_write_kernel<bf16_t>, vgrid, block, 0, stream,
                                (const bf16_t*)qkv, (bf16_t*)v_cache, positions, token_slot,
-                               block_table, table_stride, page_size, tokens, nq, nkv, d);
+                               block_table, table_stride, page_size, tokens, nq, nkv, d, row_width, v_head0);
     } else {
         return RL_ERR_ARG;
     }

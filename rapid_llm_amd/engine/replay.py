@@ -29,7 +29,7 @@ from ..config.model_config import read_config_json
 from .step import ModelRunner, StepEntry
 
 REPLAY_PAGE_SIZE = 16
-REPLAY_MAX_LIVE = 8  # traces keep up to four requests live; slots are cheap
+REPLAY_MAX_LIVE = 4  # a trace keeps at most four requests live, so slots are used again
 
 
 def build_replay_runner(model_dir: str | Path, dtype: str, max_tokens: int) -> ModelRunner:

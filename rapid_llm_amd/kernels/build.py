@@ -11,6 +11,7 @@ Two kinds of library exist:
 * ``core``: every kernel whose code does not depend on the head size.
 * ``attn_d<D>``: the matrix-core attention kernels, compiled for one head size ``D``.
   A model compiles only the head sizes it has.
+* ``mlstm``: the matrix-memory recurrence, compiled when a model has such a mixer.
 
 There is no other implementation behind these: if ``hipcc`` is missing or a compile
 fails, loading raises.
@@ -42,6 +43,7 @@ CORE_SOURCES = (
     "gemm_rows.hip",
 )
 ATTENTION_SOURCES = ("attention_mfma.hip", "attention_f32.hip")
+MLSTM_SOURCES = ("mlstm.hip",)
 HEADERS = ("common.h", "static_entry.h")
 
 # head sizes built ahead of time by build_all(): every one the kernels take.  A fresh
@@ -210,9 +212,13 @@ def attention_library(head_dim: int, force: bool = False) -> Path:
     return compile_library(f"attn_d{head_dim}", ATTENTION_SOURCES, flags, force=force)
 
 
+def mlstm_library(force: bool = False) -> Path:
+    return compile_library("mlstm", MLSTM_SOURCES, force=force)
+
+
 def build_all(head_dims: tuple[int, ...] = DEFAULT_HEAD_DIMS, force: bool = True) -> list[Path]:
     """Compile every library (what ``__graft_entry__.build`` calls)."""
-    out = [core_library(force=force)]
+    out = [core_library(force=force), mlstm_library(force=force)]
     if not all((CSRC / s).is_file() for s in ATTENTION_SOURCES):
         return out
     with ThreadPoolExecutor(min(8, len(head_dims))) as pool:

@@ -21,6 +21,7 @@ _TAG = {torch.float32: F32, torch.bfloat16: BF16}
 
 _core: ctypes.CDLL | None = None
 _attn: dict[int, ctypes.CDLL] = {}
+_mlstm: ctypes.CDLL | None = None
 
 
 class KernelError(RuntimeError):
@@ -81,6 +82,13 @@ def attention_lib(head_dim: int) -> ctypes.CDLL:
     return lib
 
 
+def mlstm_lib() -> ctypes.CDLL:
+    global _mlstm
+    if _mlstm is None:
+        _mlstm = build.load(build.mlstm_library())
+    return _mlstm
+
+
 def _stream() -> ctypes.c_void_p:
     # the raw handle of the current stream of the current device, without the stream object
     # that ``torch.cuda.current_stream()`` builds (2.8 against 0.2 us a call, on every launch)
@@ -123,9 +131,10 @@ def _ok(code: int, what: str) -> None:
 # --------------------------------------------------------------------------- #
 
 
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, fed: Optional[torch.Tensor] = None) -> None:
-    """``out[t] = table[ids[t]]``; an id ``-(r + 1)`` takes ``fed[r]``, the token a sampling
-    kernel chose in row ``r`` of the previous step."""
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, fed: Optional[torch.Tensor] = None,
+          scale: float = 1.0) -> None:
+    """``out[t] = table[ids[t]] * scale``; an id ``-(r + 1)`` takes ``fed[r]``, the token a
+    sampling kernel chose in row ``r`` of the previous step."""
     tokens = ids.numel()
     vocab, hidden = table.shape
     _need(ids, "ids", torch.int32)
@@ -136,7 +145,7 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, fed: Option
     _ok(
         core().rl_embed(
             _p(ids), _p(fed), 0 if fed is None else fed.numel(), _p(table), _tag(table.dtype), _p(out),
-            tokens, hidden, vocab, _stream(),
+            tokens, hidden, vocab, ctypes.c_float(scale), _stream(),
         ),
         "rl_embed",
     )
@@ -179,14 +188,25 @@ def add_rmsnorm(
     )
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+GLU_ALPHA = 1.702  # the sigmoid's slope in the clamped gated activation
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, limit: float = 0.0, alpha: float = GLU_ALPHA) -> None:
+    """The gated activation of a packed ``[gate | up]`` row.  ``limit`` 0: ``silu(g) * u``.
+    ``limit > 0``: ``g' * sigmoid(alpha g') * (u' + 1)`` with ``g' = min(g, limit)`` and
+    ``u' = clamp(u, -limit, limit)``."""
     tokens, two_i = gate_up.shape
+    if limit < 0:
+        raise KernelError(f"the gated activation's limit must not be negative, got {limit}")
     if two_i % 2:
         raise KernelError(f"the packed [gate | up] row must have even width, has {two_i}")
     _need(gate_up, "gate_up")
     _need(out, "out", gate_up.dtype, (tokens, two_i // 2))
     _ok(
-        core().rl_swiglu(_p(gate_up), _p(out), tokens, two_i // 2, _tag(out.dtype), _stream()),
+        core().rl_swiglu(
+            _p(gate_up), _p(out), tokens, two_i // 2, _tag(out.dtype), ctypes.c_float(limit),
+            ctypes.c_float(alpha), _stream(),
+        ),
         "rl_swiglu",
     )
 
@@ -210,6 +230,20 @@ def add_bias(y: torch.Tensor, bias: torch.Tensor) -> None:
     _need(y, "y")
     _need(bias, "bias", torch.float32, (cols,))
     _ok(core().rl_add_bias(_p(y), _p(bias), rows, cols, _tag(y.dtype), _stream()), "rl_add_bias")
+
+
+def head_gate(y: torch.Tensor, packed: torch.Tensor, gate_col: int, heads: int, d: int) -> None:
+    """``y[t, h, :] *= sigmoid(packed[t, gate_col + h])`` in place: one gate a head, read from
+    the columns ``gate_col .. gate_col + heads`` of the mixer's packed projection."""
+    tokens = y.shape[0]
+    _need(y, "y", None, (tokens, heads * d))
+    _need(packed, "packed", y.dtype, (tokens, None))
+    if not 0 <= gate_col <= packed.shape[1] - heads:
+        raise KernelError(f"gate columns {gate_col}..{gate_col + heads} lie outside rows of {packed.shape[1]}")
+    _ok(
+        core().rl_head_gate(_p(y), _p(packed), packed.shape[1], gate_col, tokens, heads, d, _tag(y.dtype), _stream()),
+        "rl_head_gate",
+    )
 
 
 def rope_table(inv_freq: torch.Tensor, positions: int) -> tuple[torch.Tensor, torch.Tensor]:
@@ -245,6 +279,7 @@ def qknorm_rope_kvwrite(
     eps: float,
     max_position: int,
     pairing: str = "half_split",
+    value_head0: Optional[int] = None,
 ) -> None:
     """Norm + rotate q and k, write k and v to the cache pages (skipped when the caches
     are ``None``: a layer that reads another layer's cache).  ``q_out`` ``None``: the query
@@ -252,11 +287,24 @@ def qknorm_rope_kvwrite(
     :func:`attention_prepares_queries`).  ``max_position`` is the
     largest position in the batch, checked against the rotation table and block table.
     The tables' width says how many channels rotate (``2 * cos.shape[1]``, the first of a
-    head), ``pairing`` which of them form a pair (:data:`ROTARY_PAIRINGS`)."""
+    head), ``pairing`` which of them form a pair (:data:`ROTARY_PAIRINGS`).
+
+    A packed row holds the query heads, then the key heads, and the value heads from head
+    ``value_head0`` on (default ``nq + nkv``, right behind the keys; ``nq``: the values are the
+    keys as projected, before the rotation); it may be wider than that (columns of the same
+    product that another kernel reads)."""
     if pairing not in ROTARY_PAIRINGS:
         raise KernelError(f"rotation pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
     tokens = qkv.shape[0]
-    _need(qkv, "qkv", None, (tokens, (nq + 2 * nkv) * d))
+    if value_head0 is None:
+        value_head0 = nq + nkv
+    _need(qkv, "qkv", None, (tokens, None))
+    row_width = qkv.shape[1]
+    if value_head0 < 0 or row_width < (max(value_head0, nq) + nkv) * d or row_width % 8:
+        raise KernelError(
+            f"packed rows of {row_width} columns do not hold {nq} query, {nkv} key and {nkv} value heads "
+            f"of {d} (values from head {value_head0}) in whole groups of 8 columns"
+        )
     if q_out is not None:
         _need(q_out, "q_out", qkv.dtype, (tokens, nq * d))
     _need(positions, "positions", torch.int32, (tokens,))
@@ -291,7 +339,7 @@ def qknorm_rope_kvwrite(
             _p(qkv), _p(q_out), _p(k_cache), _p(v_cache), _p(q_norm_w), _p(k_norm_w), _p(cos),
             _p(sin), _p(positions), _p(token_slot), _p(block_table), block_table.stride(0),
             page_size, tokens, nq, nkv, d, half, ROTARY_PAIRINGS[pairing], ctypes.c_float(eps), int(write),
-            _tag(qkv.dtype), _stream(),
+            row_width, value_head0, _tag(qkv.dtype), _stream(),
         ),
         "rl_qknorm_rope_kvwrite",
     )
@@ -1262,3 +1310,90 @@ def decode_attention_fused(
              v_cache if write_cache else None, eps)
     _decode_launch(lib, plan, ctx, qkv, k_cache, v_cache, out, block_table, page_size, nq, nkv, d,
                    window, scale, fused)
+
+
+# --------------------------------------------------------------------------- #
+# matrix-memory recurrence
+# --------------------------------------------------------------------------- #
+MLSTM_MAX_KEY_DIM = 256  # the scan stages a token's query and key of one head in LDS
+
+
+def mlstm(
+    packed: torch.Tensor,
+    columns: tuple[int, int, int, int],
+    gate_pre: torch.Tensor,
+    gate_bias: Optional[torch.Tensor],
+    norm_weight: torch.Tensor,
+    out: torch.Tensor,
+    ctx,
+    S: torch.Tensor,
+    n: torch.Tensor,
+    m: torch.Tensor,
+    heads: int,
+    dk: int,
+    dv: int,
+    cap: float,
+    eps: float,
+) -> None:
+    """The matrix-memory mixer between its projections and its output projection.
+
+    ``packed [T, width]`` holds, from the columns ``columns = (q, k, v, g)`` on, every token's
+    query and key heads (``heads * dk`` each), value heads and output gates (``heads * dv``
+    each); ``gate_pre [T, 2 * heads]`` float32 the pre-activations of the input gates, then of
+    the forget gates (``gate_bias`` is added to them).  The per-request state ``S [slots, heads,
+    dk, dv]``, ``n [slots, heads, dk]``, ``m [slots, heads]`` (float32) is read at the rows
+    ``ctx.seq_slots`` and left as it is after each request's last token of the step.
+    ``out [T, heads * dv]``: every head's output divided by its root mean square, times
+    ``norm_weight``, times the sigmoid of the output gate."""
+    tokens, width = packed.shape
+    q_col, k_col, v_col, g_col = (int(c) for c in columns)
+    _need(packed, "packed projections")
+    _need(gate_pre, "gate pre-activations", torch.float32, (tokens, 2 * heads))
+    if gate_bias is not None:
+        _need(gate_bias, "gate bias", torch.float32, (2 * heads,))
+    _need(norm_weight, "head norm weight", torch.float32, (heads * dv,))
+    _need(out, "out", packed.dtype, (tokens, heads * dv))
+    slots = S.shape[0]
+    _need(S, "state S", torch.float32, (slots, heads, dk, dv))
+    _need(n, "state n", torch.float32, (slots, heads, dk))
+    _need(m, "state m", torch.float32, (slots, heads))
+    _need(ctx.cu_seqlens, "cu_seqlens", torch.int32, (ctx.num_seqs + 1,))
+    _need(ctx.seq_slots, "seq_slots", torch.int32, (ctx.num_seqs,))
+    if not 1 <= dk <= MLSTM_MAX_KEY_DIM:
+        raise KernelError(f"the recurrence takes key sizes up to {MLSTM_MAX_KEY_DIM}, got {dk}")
+    for name, col, size in (("q", q_col, heads * dk), ("k", k_col, heads * dk), ("v", v_col, heads * dv),
+                            ("g", g_col, heads * dv)):
+        if col < 0 or col + size > width:
+            raise KernelError(f"columns {col}..{col + size} of {name} lie outside packed rows of {width}")
+    if ctx.h_seq_slots and max(ctx.h_seq_slots) >= slots:
+        raise KernelError(f"slot {max(ctx.h_seq_slots)} is outside a state of {slots} slots")
+    if sum(ctx.h_seq_lens) != tokens:
+        raise KernelError(f"the step's requests bring {sum(ctx.h_seq_lens)} tokens, the rows are {tokens}")
+    lib = mlstm_lib()
+    dev = packed.device
+    log_keep = torch.empty((tokens, heads), dtype=torch.float32, device=dev)
+    log_take = torch.empty_like(log_keep)
+    m_tok = torch.empty_like(log_keep)
+    raw = torch.empty((tokens, heads, dv + 1), dtype=torch.float32, device=dev)
+    _ok(
+        lib.rl_mlstm_gates(
+            _p(gate_pre), _p(gate_bias), _p(ctx.cu_seqlens), _p(ctx.seq_slots), _p(m), _p(log_keep),
+            _p(log_take), _p(m_tok), ctx.num_seqs, heads, ctypes.c_float(cap), _stream(),
+        ),
+        "rl_mlstm_gates",
+    )
+    _ok(
+        lib.rl_mlstm_scan(
+            _p(packed), width, q_col, k_col, v_col, _p(log_keep), _p(log_take), _p(ctx.cu_seqlens),
+            _p(ctx.seq_slots), _p(S), _p(n), _p(raw), ctx.num_seqs, heads, dk, dv,
+            ctypes.c_float(float(dk) ** -0.5), _tag(packed.dtype), _stream(),
+        ),
+        "rl_mlstm_scan",
+    )
+    _ok(
+        lib.rl_mlstm_finish(
+            _p(raw), _p(m_tok), _p(packed), width, g_col, _p(norm_weight), _p(out), tokens, heads, dv,
+            ctypes.c_float(eps), _tag(packed.dtype), _stream(),
+        ),
+        "rl_mlstm_finish",
+    )

@@ -24,6 +24,7 @@ from ..parts.base import (
     ParamSpec,
 )
 from ..parts.lazy import plain, run_norm
+from ..parts.offsets import StreamOffsetTable
 from .spec import ModelSpec
 
 
@@ -39,6 +40,13 @@ class CausalLM:
         for li in self.order:
             if not 0 <= li < len(spec.layers):
                 raise ValueError(f"run order names layer {li}; the model has {len(spec.layers)}")
+        self.offsets = None
+        if spec.stream_offsets is not None:
+            so = spec.stream_offsets
+            for place in so.places:
+                if not 0 <= place < len(self.order):
+                    raise ValueError(f"a stream offset names place {place} of a run order of {len(self.order)}")
+            self.offsets = StreamOffsetTable(so.checkpoint_name, so.places, spec.hidden_size, name="stream_offsets")
         self._positions: dict[str, object] = {}
         self.blocks = []
         for i, layer in enumerate(spec.layers):
@@ -50,13 +58,17 @@ class CausalLM:
             mixer = MIXERS.create(
                 layer.mixer.kind, **layer.mixer.params, position=position, name=f"layers.{i}.mixer"
             )
-            ff = FEED_FORWARDS.create(
-                layer.feed_forward.kind, **layer.feed_forward.params, name=f"layers.{i}.ff"
-            )
+            if (layer.feed_forward is None) != (layer.feed_forward_norm is None):
+                raise ValueError(f"layer {i}: a feed-forward and its norm come together or not at all")
+            ff = n2 = None
+            if layer.feed_forward is not None:
+                ff = FEED_FORWARDS.create(
+                    layer.feed_forward.kind, **layer.feed_forward.params, name=f"layers.{i}.ff"
+                )
+                n2 = NORMS.create(
+                    layer.feed_forward_norm.kind, **layer.feed_forward_norm.params, name=f"layers.{i}.ff_norm"
+                )
             n1 = NORMS.create(layer.mixer_norm.kind, **layer.mixer_norm.params, name=f"layers.{i}.mixer_norm")
-            n2 = NORMS.create(
-                layer.feed_forward_norm.kind, **layer.feed_forward_norm.params, name=f"layers.{i}.ff_norm"
-            )
             self.blocks.append(
                 BLOCKS.create(
                     layer.block.kind,
@@ -75,6 +87,8 @@ class CausalLM:
             yield from block.parts()
         yield self.final_norm
         yield self.output
+        if self.offsets is not None:
+            yield self.offsets
         yield from self._positions.values()
 
     def param_specs(self) -> list[ParamSpec]:
@@ -122,6 +136,8 @@ class CausalLM:
         delta = None
         for place, li in enumerate(self.order):
             block = self.blocks[li]
+            if self.offsets is not None:
+                self.offsets.add(residual, place)
             if not getattr(block, "accepts_deferred", False):
                 delta = plain(delta)
             delta = block.forward(residual, delta, ctx, caches[place])

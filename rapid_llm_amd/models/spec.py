@@ -4,7 +4,9 @@ An architecture's builder turns its typed configuration into a :class:`ModelSpec
 which mixer, feed-forward, norms and block each layer has (chosen layer by layer, each
 with its own parameters), which embedding and output projection stand at its two ends,
 and the order in which layers run.  The order is data too: ``run_order`` may name a layer
-twice, and a layer may read another layer's cache (``LayerSpec.share_cache_with``).
+twice, and a layer may read another layer's cache (``LayerSpec.share_cache_with``).  A layer
+may lack the feed-forward sub-layer, and learned vectors may be added to the stream at given
+places of the order (``ModelSpec.stream_offsets``).
 """
 
 from __future__ import annotations
@@ -33,9 +35,9 @@ class LayerSpec:
     """One layer: parts by kind and parameters, plus where its tensors sit in the checkpoint."""
 
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: PartSpec | None  # None: the layer has the mixer's sub-layer only
     mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    feed_forward_norm: PartSpec | None
     block: PartSpec = PartSpec("prenorm")
     position: PartSpec = PartSpec("none")
     checkpoint_prefix: str = ""
@@ -47,6 +49,24 @@ def token_embedding(vocab_size: int, hidden_size: int, checkpoint_name: str) -> 
     return PartSpec(
         "token_embedding", {"vocab_size": vocab_size, "hidden_size": hidden_size, "checkpoint_name": checkpoint_name}
     )
+
+
+def token_embedding_scaled(vocab_size: int, hidden_size: int, checkpoint_name: str, scale: float) -> PartSpec:
+    """The table lookup times a constant."""
+    return PartSpec(
+        "token_embedding",
+        {"vocab_size": vocab_size, "hidden_size": hidden_size, "checkpoint_name": checkpoint_name, "scale": scale},
+    )
+
+
+@dataclass(frozen=True)
+class StreamOffsets:
+    """Learned vectors added to the residual stream: row ``t`` of the checkpoint tensor
+    ``checkpoint_name`` (``[len(places), hidden]``) is added to every token's stream right
+    before the layer at place ``places[t]`` of the run order runs."""
+
+    checkpoint_name: str
+    places: tuple[int, ...]
 
 
 def linear_output(vocab_size: int, hidden_size: int, checkpoint_name: str, tied: bool) -> PartSpec:
@@ -70,6 +90,7 @@ class ModelSpec:
     run_order: tuple[int, ...] | None = None  # None: 0..len(layers)-1
     ignore_tensors: tuple[IgnoreRule, ...] = ()
     max_position: int = 0  # largest position the architecture is defined for (0: unbounded)
+    stream_offsets: StreamOffsets | None = None
 
     def order(self) -> tuple[int, ...]:
         return self.run_order if self.run_order is not None else tuple(range(len(self.layers)))

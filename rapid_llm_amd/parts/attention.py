@@ -13,6 +13,13 @@ Keys and values are always read back from the pages, also for the tokens of the 
 step, so that one code path serves whole prompts, portions and single decoded tokens
 (the reference switches kernels by phase, attention.py:179-240).  ``window`` > 0 limits a
 query at position p to keys ``[p - window + 1, p]`` (rapid_llm/engine/kv_cache_spec.py:203-222).
+
+Two options change what the packed projection holds.  ``values="keys"``: there is no value
+projection, a token's values are its keys as projected, before the rotation; the packed row is
+``[q | k]`` and the cache write reads the values from the key columns.  ``head_gate_name``: a
+projection of one number per query head rides in the same product (rows behind the keys and
+values, padded to a multiple of 8), and every head's output is multiplied by the sigmoid of its
+number before the output projection.
 """
 
 from __future__ import annotations
@@ -49,6 +56,9 @@ class GQAAttention(Mixer):
         k_norm_name: str = "k_norm.weight",
         qkv_bias: bool = False,
         o_bias: bool = False,
+        values: str = "own",
+        head_gate_name: str | None = None,
+        bias_names: dict[str, str] | None = None,
     ) -> None:
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not divisible by {num_kv_heads} kv heads")
@@ -69,10 +79,22 @@ class GQAAttention(Mixer):
             raise ValueError(
                 f"the attention kernels rotate pairs as {sorted(ops.ROTARY_PAIRINGS)}, not as {pairing!r}"
             )
+        if values not in ("own", "keys"):
+            raise ValueError(f"the values are the mixer's 'own' projection or its 'keys', not {values!r}")
         self.scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(head_dim)
         self.name = name
-        self.names = dict(q=q_name, k=k_name, v=v_name, o=o_name, qn=q_norm_name, kn=k_norm_name)
-        self.qkv = Linear(hidden_size, (num_heads + 2 * num_kv_heads) * head_dim)
+        self.names = dict(q=q_name, k=k_name, v=v_name, o=o_name, qn=q_norm_name, kn=k_norm_name,
+                          g=head_gate_name)
+        self.bias_names = dict(bias_names or {})
+        self.values_are_keys = values == "keys"
+        # the packed row: query heads, key heads, value heads unless they are the keys, then
+        # one gate per query head, padded so that rows stay whole groups of 8 columns
+        self.value_head0 = num_heads if self.values_are_keys else num_heads + num_kv_heads
+        self.qkv_rows = (num_heads + (1 if self.values_are_keys else 2) * num_kv_heads) * head_dim
+        self.gate_rows = num_heads if head_gate_name else 0
+        self.gate_pad = -self.gate_rows % 8
+        self.plain_row = not self.values_are_keys and not self.gate_rows
+        self.qkv = Linear(hidden_size, self.qkv_rows + self.gate_rows + self.gate_pad)
         self.o = Linear(num_heads * head_dim, hidden_size)
         self.q_norm_w = self.k_norm_w = None
         # Qwen3 has neither (rapid_llm/models/qwen3.py:16-18: qkv_bias=False); architectures of the
@@ -84,13 +106,15 @@ class GQAAttention(Mixer):
     def param_specs(self) -> list[ParamSpec]:
         p, n = self.prefix, self.names
         q_rows, kv_rows = self.nq * self.d, self.nkv * self.d
+        packed = [Source(p + n["q"], q_rows), Source(p + n["k"], kv_rows)]
+        if not self.values_are_keys:
+            packed.append(Source(p + n["v"], kv_rows))
+        if self.gate_rows:
+            packed.append(Source(p + n["g"], self.gate_rows))
+        if self.gate_pad:
+            packed.append(Source("", self.gate_pad))  # rows of zeros
         specs = [
-            ParamSpec(
-                self.name + ".qkv",
-                (q_rows + 2 * kv_rows, self.hidden_size),
-                "matrix",
-                (Source(p + n["q"], q_rows), Source(p + n["k"], kv_rows), Source(p + n["v"], kv_rows)),
-            ),
+            ParamSpec(self.name + ".qkv", (self.qkv.out_features, self.hidden_size), "matrix", tuple(packed)),
             ParamSpec(self.name + ".o", (self.hidden_size, q_rows), "matrix", (Source(p + n["o"], self.hidden_size),)),
         ]
         if self.qk_norm_eps is not None:
@@ -99,18 +123,22 @@ class GQAAttention(Mixer):
                 ParamSpec(self.name + ".k_norm", (self.d,), "vector", (Source(p + n["kn"], self.d),), init="norm"),
             ]
 
-        def bias_of(weight_name: str) -> str:
+        def bias_of(which: str) -> str:
+            if which in self.bias_names:
+                return self.bias_names[which]
+            weight_name = n[which]
             return weight_name[: -len("weight")] + "bias" if weight_name.endswith("weight") else weight_name + ".bias"
 
         if self.qkv_bias:
-            specs.append(ParamSpec(
-                self.name + ".qkv_bias", (q_rows + 2 * kv_rows,), "vector",
-                (Source(p + bias_of(n["q"]), q_rows), Source(p + bias_of(n["k"]), kv_rows),
-                 Source(p + bias_of(n["v"]), kv_rows)),
-            ))
+            biases = [Source(p + bias_of("q"), q_rows), Source(p + bias_of("k"), kv_rows)]
+            if not self.values_are_keys:
+                biases.append(Source(p + bias_of("v"), kv_rows))
+            if self.gate_rows + self.gate_pad:
+                biases.append(Source("", self.gate_rows + self.gate_pad))  # the gates have none
+            specs.append(ParamSpec(self.name + ".qkv_bias", (self.qkv.out_features,), "vector", tuple(biases)))
         if self.o_bias:
             specs.append(ParamSpec(
-                self.name + ".o_bias", (self.hidden_size,), "vector", (Source(p + bias_of(n["o"]), self.hidden_size),)
+                self.name + ".o_bias", (self.hidden_size,), "vector", (Source(p + bias_of("o"), self.hidden_size),)
             ))
         return specs
 
@@ -145,7 +173,9 @@ class GQAAttention(Mixer):
         out = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
         rotary_half = cos.shape[1] if cos is not None else 0
         pairing = getattr(pos_enc, "pairing", "half_split") if cos is not None else "half_split"
-        if ops.decode_attention_fusable(ctx, qkv.dtype, self.nq // self.nkv, self.d, rotary_half, pairing):
+        if self.plain_row and ops.decode_attention_fusable(
+            ctx, qkv.dtype, self.nq // self.nkv, self.d, rotary_half, pairing
+        ):
             # a step of single tokens: norm, rotation, cache write and attention in one kernel
             ops.decode_attention_fused(
                 qkv, cache.k, cache.v, out, ctx, table, cache.page_size, self.nq, self.nkv, self.d,
@@ -154,7 +184,7 @@ class GQAAttention(Mixer):
             return self.o.deferred(out, ctx)
         # where the attention kernels can finish the query heads as they read them, only the keys
         # and values are prepared here, and the queries are never written out
-        in_kernel = ops.attention_prepares_queries(qkv.dtype, self.d, rotary_half, pairing)
+        in_kernel = self.plain_row and ops.attention_prepares_queries(qkv.dtype, self.d, rotary_half, pairing)
         q = None if in_kernel else torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
         ops.qknorm_rope_kvwrite(
             qkv, q,
@@ -162,13 +192,15 @@ class GQAAttention(Mixer):
             cache.v if cache.owns_pages else None,
             self.q_norm_w, self.k_norm_w, cos, sin,
             ctx.positions, ctx.token_slot, table, cache.page_size,
-            self.nq, self.nkv, self.d, eps, ctx.max_position, pairing,
+            self.nq, self.nkv, self.d, eps, ctx.max_position, pairing, self.value_head0,
         )
         ops.paged_attention(
             qkv if in_kernel else q, cache.k, cache.v, out, ctx, table, cache.page_size,
             self.nq, self.nkv, self.d, self.window, self.scale,
             prepare=(self.q_norm_w, cos, sin, eps) if in_kernel else None,
         )
+        if self.gate_rows:
+            ops.head_gate(out, qkv, self.qkv_rows, self.nq, self.d)
         return self.o.deferred(out, ctx)
 
 

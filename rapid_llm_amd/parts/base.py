@@ -38,7 +38,9 @@ if TYPE_CHECKING:  # pragma: no cover
 
 @dataclass(frozen=True)
 class Source:
-    """One checkpoint tensor feeding ``rows`` rows (dim 0) of a parameter."""
+    """One checkpoint tensor feeding ``rows`` rows (dim 0) of a parameter.  An empty name
+    stands for ``rows`` rows of zeros that no checkpoint tensor feeds (padding of a packed
+    matrix to a width its kernels take)."""
 
     name: str
     rows: int
@@ -57,6 +59,8 @@ class ParamSpec:
         checkpoint stores in 32-bit stays 32-bit.
       * ``"vector"``: small per-channel weights (norms); always held in float32, which
         represents a bfloat16 checkpoint value exactly.
+      * ``"matrix_f32"``: a matrix that is held in float32 in every engine, so that its
+        product is a true 32-bit one (the gates of a recurrence).
       * ``"table"``: integer lookup tables, held as int32.
     ``fallback`` names another parameter whose tensor is shared when the checkpoint has
     none of this one's sources (a tied output projection).

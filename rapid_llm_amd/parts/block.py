@@ -1,4 +1,5 @@
-"""Pre-norm arrangement: ``r += mixer(norm(r)); r += feed_forward(norm(r))``.
+"""Pre-norm arrangement: ``r += mixer(norm(r)); r += feed_forward(norm(r))``; a layer
+without a feed-forward has the first sub-layer only.
 
 The add of each sub-layer's output is carried forward as ``delta`` and happens inside the
 next norm kernel, as the reference threads ``(hidden, residual)`` through its layers
@@ -22,11 +23,15 @@ class PreNormBlock(Block):
         self.feed_forward_norm = feed_forward_norm
 
     def parts(self):
+        if self.feed_forward is None:
+            return (self.mixer_norm, self.mixer)
         return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
 
     def forward(self, residual, delta, ctx, cache):
         x = run_norm(self.mixer_norm, residual, delta, ctx, consumer=self.mixer)
         a = self.mixer.forward(x, ctx, cache)
+        if self.feed_forward is None:
+            return a
         x = run_norm(self.feed_forward_norm, residual, a, ctx, consumer=self.feed_forward)
         return self.feed_forward.forward(x, ctx)
 

@@ -17,8 +17,10 @@ from .linear import Linear
 class TokenEmbedding(Embedding):
     replayable = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, checkpoint_name: str, name: str = "embed") -> None:
+    def __init__(self, vocab_size: int, hidden_size: int, checkpoint_name: str, name: str = "embed",
+                 scale: float = 1.0) -> None:
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
+        self.scale = float(scale)  # every row is multiplied by it on its way into the stream
         self.checkpoint_name = checkpoint_name
         self.name = name
         self.table: torch.Tensor | None = None
@@ -39,7 +41,7 @@ class TokenEmbedding(Embedding):
     def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
         """Rows of the table for the ids; an id ``-(r + 1)`` takes ``ctx.fed_tokens[r]``."""
         out = torch.empty((token_ids.numel(), self.hidden_size), dtype=torch.float32, device=token_ids.device)
-        ops.embed(token_ids, self.table, out, getattr(ctx, "fed_tokens", None))
+        ops.embed(token_ids, self.table, out, getattr(ctx, "fed_tokens", None), self.scale)
         return out
 
 

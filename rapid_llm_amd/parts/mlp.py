@@ -1,4 +1,6 @@
-"""Dense SwiGLU feed-forward: ``down(silu(gate(x)) * up(x))``.
+"""Dense gated feed-forward: ``down(act(gate(x), up(x)))`` with ``act(g, u) = silu(g) * u``
+(SwiGLU), or, with a ``limit``, the clamped variant ``g' * sigmoid(alpha * g') * (u' + 1)`` where
+``g' = min(g, limit)`` and ``u' = clamp(u, -limit, limit)``.
 
 Gate and up are one packed matrix ``[2I, H]`` with rows ``[gate | up]``
 (rapid_llm/models/base.py:401-404, rapid_llm/modules/linear.py:157-172), so one product
@@ -27,7 +29,12 @@ class SwiGLU(FeedForward):
         gate_name: str = "gate_proj.weight",
         up_name: str = "up_proj.weight",
         down_name: str = "down_proj.weight",
+        limit: float = 0.0,
+        alpha: float = ops.GLU_ALPHA,
     ) -> None:
+        if limit < 0:
+            raise ValueError(f"the gated activation's limit must not be negative, got {limit}")
+        self.limit, self.alpha = float(limit), float(alpha)
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.prefix = checkpoint_prefix
@@ -54,15 +61,16 @@ class SwiGLU(FeedForward):
 
     def forward(self, x, ctx):
         w = self.gate_up.weight
-        if w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
+        if w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and not self.limit:
             # few rows: product and activation in one kernel
             act = ops.gemm_bf16_swiglu(x.rows, w, scaled=x) if isinstance(x, ScaledRows) else ops.gemm_bf16_swiglu(x, w)
             if act is not None:
                 return self.down.deferred(act, ctx)
         gu = self.gate_up(x)
         act = torch.empty((x.shape[0], self.intermediate_size), dtype=gu.dtype, device=x.device)
-        ops.swiglu(gu, act)
+        ops.swiglu(gu, act, self.limit, self.alpha)
         return self.down.deferred(act, ctx)
 
 
 FEED_FORWARDS.register("swiglu", SwiGLU)
+FEED_FORWARDS.register("gated", SwiGLU)  # the same part under the name that fits either activation

@@ -75,7 +75,7 @@ def iterate_checkpoint(model_dir: str | Path) -> Iterator[tuple[str, torch.Tenso
 def storage_dtype(role: str, stored: torch.dtype, engine_dtype: torch.dtype) -> torch.dtype:
     if role == "table":
         return torch.int32
-    if role == "vector":
+    if role in ("vector", "matrix_f32"):
         return torch.float32
     if engine_dtype == torch.float32:
         return torch.float32
@@ -109,6 +109,9 @@ def load_params(
     for spec in specs:
         offset = 0
         for src in spec.sources:
+            if not src.name:  # rows of zeros that no checkpoint tensor feeds
+                offset += src.rows
+                continue
             if src.name in by_source:
                 other.append(f"checkpoint tensor {src.name!r} is claimed by two parameters")
             by_source[src.name] = (spec, offset, src.rows)
@@ -150,7 +153,8 @@ def load_params(
         dest = out.get(spec.name)
         dtype = storage_dtype(spec.role, tensor.dtype, engine_dtype)
         if dest is None:
-            dest = torch.empty(spec.shape, dtype=dtype, device=device)
+            padded = any(not s.name for s in spec.sources)
+            dest = (torch.zeros if padded else torch.empty)(spec.shape, dtype=dtype, device=device)
             out[spec.name] = dest
         elif dest.dtype != dtype:
             # blocks of one fused matrix stored in different widths: keep the wider
@@ -161,10 +165,11 @@ def load_params(
 
     missing: list[str] = []
     for spec in specs:
-        absent = [s.name for s in spec.sources if s.name not in seen]
+        named = [s for s in spec.sources if s.name]
+        absent = [s.name for s in named if s.name not in seen]
         if not absent:
             continue
-        if len(absent) == len(spec.sources) and spec.fallback is not None:
+        if len(absent) == len(named) and spec.fallback is not None:
             continue  # resolved below by sharing
         missing.extend(f"{n} (for parameter {spec.name!r})" for n in absent)
     if missing or unexpected or wrong or other:

@@ -52,6 +52,8 @@ def random_checkpoint_tensors(
         if spec.fallback is not None:
             continue  # shared with another parameter: the checkpoint ships none
         for src in spec.sources:
+            if not src.name:
+                continue  # rows of zeros: the checkpoint ships nothing for them
             shape = (src.rows, *spec.shape[1:])
             t = _draw(shape, spec.init, gen, std, norm_std)
             out[src.name] = t.to(_STORE[dtype]) if spec.role != "table" else t.to(torch.int32)
@@ -108,6 +110,8 @@ def random_params(
             continue
         if spec.role == "vector":
             out[spec.name] = _draw(spec.shape, spec.init, gen, std, norm_std, device)
+        elif spec.role == "matrix_f32":
+            out[spec.name] = torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
         elif spec.role == "table":
             out[spec.name] = torch.zeros(spec.shape, dtype=torch.int32, device=device)
         else:
@@ -117,4 +121,10 @@ def random_params(
     for spec in specs:
         if spec.fallback is not None:
             out[spec.name] = out[spec.fallback]
+            continue
+        offset = 0
+        for src in spec.sources:
+            if not src.name:  # rows no checkpoint tensor would feed are zeros here too
+                out[spec.name][offset : offset + src.rows] = 0
+            offset += src.rows
     return out
