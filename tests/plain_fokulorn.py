@@ -69,24 +69,30 @@ def plain_softmax_attention(q, k, v, scale: float, window: int | None) -> torch.
     return out
 
 
-def plain_keyvalue_attention(h, w, p, cfg, positions=None) -> torch.Tensor:
+def _same(x):
+    return x
+
+
+def plain_keyvalue_attention(h, w, p, cfg, positions=None, cast=_same) -> torch.Tensor:
     """The softmax mixer whose values are its keys: ``v`` is the key projection before the
-    rotation.  ``w(name)`` returns the mixer's tensor ``name``; ``cfg`` is its ``mixer`` dict."""
+    rotation.  ``w(name)`` returns the mixer's tensor ``name``; ``cfg`` is its ``mixer`` dict.
+    ``cast`` rounds what an engine would store in its compute type (projections, rotated
+    heads, the heads' outputs)."""
     t = h.shape[0]
     heads, kv, dk = cfg["heads"], cfg["kv_heads"], cfg["dim"]
     positions = torch.arange(t) if positions is None else positions
-    q = (h @ w("q").T + w("q.b")).view(t, heads, dk)
-    k = (h @ w("k").T + w("k.b")).view(t, kv, dk)
+    q = cast(h @ w("q").T + w("q.b")).view(t, heads, dk)
+    k = cast(h @ w("k").T + w("k.b")).view(t, kv, dk)
     v = k
     rot = cfg.get("rot")
     if rot:
-        q = plain_rotate_interleaved(q, positions, rot["dims"], rot["base"])
-        k = plain_rotate_interleaved(k, positions, rot["dims"], rot["base"])
+        q = cast(plain_rotate_interleaved(q, positions, rot["dims"], rot["base"]))
+        k = cast(plain_rotate_interleaved(k, positions, rot["dims"], rot["base"]))
     mask = cfg.get("mask")
-    o = plain_softmax_attention(q, k, v, cfg["scale"], mask["size"] if mask else None)
-    gate = torch.sigmoid(h @ w("g").T)  # [T, H]: one number a head
-    o = o * gate[:, :, None]
-    return o.reshape(t, heads * v.shape[-1]) @ w("o").T
+    o = cast(plain_softmax_attention(q, k, v, cfg["scale"], mask["size"] if mask else None))
+    gate = torch.sigmoid(cast(h @ w("g").T))  # [T, H]: one number a head
+    o = cast(o * gate[:, :, None])
+    return cast(o.reshape(t, heads * v.shape[-1]) @ w("o").T)
 
 
 def plain_mlstm_gates(h, w, cap: float):
@@ -123,28 +129,29 @@ def plain_mlstm_scan(q, k, v, i, f, state=None):
     return out, (S, n, m)
 
 
-def plain_mlstm(h, w, cfg, eps: float) -> torch.Tensor:
+def plain_mlstm(h, w, cfg, eps: float, cast=_same) -> torch.Tensor:
     """The matrix-memory mixer: projections, gates, recurrence, per-head unit RMS, the
-    weight over all heads, the sigmoid gate, the output projection."""
+    weight over all heads, the sigmoid gate, the output projection.  ``cast`` rounds the
+    projections and the finished heads; gates, state and recurrence are never rounded."""
     t = h.shape[0]
     heads, dk, dv = cfg["heads"], cfg["dim"], cfg["vdim"]
-    q = (h @ w("q").T).view(t, heads, dk) * dk ** -0.5
-    k = (h @ w("k").T).view(t, heads, dk)
-    v = (h @ w("v").T).view(t, heads, dv)
+    q = cast(h @ w("q").T).view(t, heads, dk) * dk ** -0.5
+    k = cast(h @ w("k").T).view(t, heads, dk)
+    v = cast(h @ w("v").T).view(t, heads, dv)
     i, f = plain_mlstm_gates(h, w, cfg["gate_cap"])
     o, _ = plain_mlstm_scan(q, k, v, i, f)
     o = plain_rms(o, eps).reshape(t, heads * dv) * w("norm")
-    o = o * torch.sigmoid(h @ w("g").T)
-    return o @ w("o").T
+    o = cast(o * torch.sigmoid(cast(h @ w("g").T)))
+    return cast(o @ w("o").T)
 
 
-def plain_clamped_glu(h, w, cfg) -> torch.Tensor:
+def plain_clamped_glu(h, w, cfg, cast=_same) -> torch.Tensor:
     """``down(g * sigmoid(1.702 g) * (u + 1))`` with ``g = min(gate(h), limit)`` and
     ``u = clamp(up(h), -limit, limit)``."""
     limit = cfg["limit"]
-    g = (h @ w("gate").T).clamp(max=limit)
-    u = (h @ w("up").T).clamp(-limit, limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w("down").T
+    g = cast(h @ w("gate").T).clamp(max=limit)
+    u = cast(h @ w("up").T).clamp(-limit, limit)
+    return cast(cast(g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w("down").T)
 
 
 # --------------------------------------------------------------------------- #
@@ -167,9 +174,11 @@ def plain_run_order(cfg) -> list[tuple[int, int | None]]:
     return order
 
 
-def plain_forward(cfg, weights, tokens, dtype=torch.float32, streams: list | None = None) -> torch.Tensor:
+def plain_forward(cfg, weights, tokens, dtype=torch.float32, streams: list | None = None, cast=_same) -> torch.Tensor:
     """Logits ``[T, vocab]`` of one sequence.  ``streams``, when given, receives the residual
-    stream after every layer run."""
+    stream after every layer run.  ``cast`` rounds every activation that an engine stores in
+    its compute type (never the residual stream, gates or recurrent state): with a bfloat16
+    rounding it measures what rounding alone does to the logits."""
     W = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     eps = cfg["norm"]["eps"]
     x = W["embed"][torch.as_tensor(tokens, dtype=torch.long)] * cfg["embedding"]["scale"]
@@ -185,18 +194,18 @@ def plain_forward(cfg, weights, tokens, dtype=torch.float32, streams: list | Non
         def mlp(name, pre=pre):
             return W[pre + "mlp." + name]
 
-        h = plain_rmsnorm(x, W[pre + "norm1"], eps)
+        h = cast(plain_rmsnorm(x, W[pre + "norm1"], eps))
         if spec["type"] == "attention":
-            x = x + plain_keyvalue_attention(h, mix, None, spec["mixer"])
+            x = x + plain_keyvalue_attention(h, mix, None, spec["mixer"], cast=cast)
         elif spec["type"] == "mlstm":
-            x = x + plain_mlstm(h, mix, spec["mixer"], eps)
+            x = x + plain_mlstm(h, mix, spec["mixer"], eps, cast=cast)
         else:
             raise ValueError(f"unknown mixer {spec['type']!r}")
         if spec.get("mlp") is not None:
-            h = plain_rmsnorm(x, W[pre + "norm2"], eps)
-            x = x + plain_clamped_glu(h, mlp, spec["mlp"])
+            h = cast(plain_rmsnorm(x, W[pre + "norm2"], eps))
+            x = x + plain_clamped_glu(h, mlp, spec["mlp"], cast=cast)
         if streams is not None:
             streams.append(x.clone())
-    x = plain_rmsnorm(x, W["final.norm"], eps)
+    x = cast(plain_rmsnorm(x, W["final.norm"], eps))
     return x @ W["head"].T
 
