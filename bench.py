@@ -3,6 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bfloat16]
                     [--shape NAME] [--batch B] [--prompt-len T] [--context C]
     python bench.py --workload qwen3-0.6b-256 | qwen3-32b-32
+    python bench.py --design fokulorn [--design-size 2b,8b]
 
 A "step" is one decode step of the whole batch through the engine's step function and the
 greedy sampling kernel, tokens fed back.  The default run has the layer sizes of
@@ -21,6 +22,13 @@ Qwen3-0.6B shape, 256 requests at once, prompts uniform in 64 to 1,024 tokens, 1
 generated tokens a second and the decode step's share of the HBM roofline, each measured in a
 process of its own through the continuous-batching scheduler (``--workload NAME`` runs one
 alone; ``--no-workloads`` leaves them out).
+
+``--design fokulorn`` measures another architecture of the engine, the Fokulorn decoder
+(matrix-memory recurrences beside windowed attention whose values are its keys), at layer
+sizes of real models, beside the Qwen3 decoder of the same width, depth, heads and
+feed-forward width: prefill of one prompt and decode at batch 8 through the same step
+function, and the design's own kernels alone against their rooflines.  It prints one line of
+its own and leaves the default run as it is.
 
 Metric definitions follow rapid_llm's docs/benchmark_models.md:141-149: decode tok/s is
 batch / mean step time; prefill tok/s is prompt tokens / prefill latency; both timed
@@ -274,6 +282,162 @@ def float32_points(args) -> dict:
         return {}
 
 
+# Layer sizes for ``--design fokulorn``: three recurrent layers to one of attention, the
+# attention as in the Qwen3 shape of that width, the recurrence with half the width in keys and
+# the whole width in values (heads of 128 / 256 and of 256 / 512 channels).
+DESIGN_SIZES = {
+    "2b": dict(width=2048, layers=8, heads=16, kv_heads=8, head_dim=128, ff=6144, vocab=151936,
+               mem_heads=8, mem_dk=128, mem_dv=256, window=1024),
+    "8b": dict(width=4096, layers=8, heads=32, kv_heads=8, head_dim=128, ff=12288, vocab=151936,
+               mem_heads=8, mem_dk=256, mem_dv=512, window=1024),
+}
+
+
+def fokulorn_body(z: dict) -> dict:
+    layers = []
+    for i in range(z["layers"]):
+        if i % 4 == 3:
+            layers.append({"type": "attention", "mixer": {
+                "heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["head_dim"], "vdim": z["head_dim"],
+                "scale": z["head_dim"] ** -0.5, "mask": {"size": z["window"]},
+                "rot": {"dims": z["head_dim"] // 2, "base": 10000.0}},
+                "mlp": {"kind": "dense", "ff": z["ff"], "limit": 7.0}})
+        else:
+            layers.append({"type": "mlstm", "mixer": {
+                "heads": z["mem_heads"], "dim": z["mem_dk"], "vdim": z["mem_dv"], "gate_cap": 15.0},
+                "mlp": {"kind": "dense", "ff": z["ff"], "limit": 7.0}})
+    return {"architecture": "Fokulorn", "width": z["width"], "vocab": z["vocab"], "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-6}, "layers": layers}
+
+
+def qwen3_body(z: dict) -> dict:
+    return dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=z["layers"],
+                hidden_size=z["width"], num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"],
+                head_dim=z["head_dim"], intermediate_size=z["ff"], vocab_size=z["vocab"], rope_theta=1e6,
+                rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960)
+
+
+def _time_model(body: dict, prompt_len: int, batch: int, steps: int, context: int) -> dict:
+    """Prefill of one prompt and decode at ``batch`` through ``ModelRunner.step``."""
+    import torch
+
+    from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry
+
+    pages = batch * (-(-(prompt_len + steps + 40) // 16)) + 1
+    runner = ModelRunner(body, EngineConfig(dtype="bfloat16", max_seq_len=context, page_size=16, num_pages=pages,
+                                            max_num_seqs=batch, max_num_batched_tokens=8192, seed=1234),
+                         load_format="random")
+    gen = torch.Generator().manual_seed(7)
+    vocab = runner.vocab_size
+
+    def prompt():
+        return torch.randint(0, vocab, (prompt_len,), generator=gen).tolist()
+
+    times = []
+    for _ in range(4):
+        toks = prompt()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        runner.step([StepEntry("p", toks, [prompt_len - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t)
+        runner.finish("p")
+    prefill = statistics.median(times[1:])
+    ids = [f"d{i}" for i in range(batch)]
+    for rid in ids:
+        runner.step([StepEntry(rid, prompt(), [prompt_len - 1])])
+    entries = [StepEntry(rid, [1 + i], [0]) for i, rid in enumerate(ids)]
+    for _ in range(12):
+        runner.step(entries)
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(steps):
+        runner.step(entries)
+    torch.cuda.synchronize()
+    decode = (time.perf_counter() - t) / steps
+    out = {"prefill_tok_s": round(prompt_len / prefill, 1), "prefill_ms": round(prefill * 1e3, 3),
+           "decode_tok_s": round(batch / decode, 1), "decode_ms": round(decode * 1e3, 4)}
+    del runner
+    torch.cuda.empty_cache()
+    return out
+
+
+def _time_kernels(z: dict, prompt_len: int, batch: int) -> dict:
+    """The design's own kernels alone, microseconds and share of the roofline each: the
+    recurrence over one prompt (float32 matrix rate) and over ``batch`` single tokens (bytes
+    of state read and written), and the two row-wise kernels (bytes)."""
+    import types
+
+    import torch
+
+    from rapid_llm_amd.kernels import ops
+
+    h, dk, dv = z["mem_heads"], z["mem_dk"], z["mem_dv"]
+    width = 2 * h * dk + 2 * h * dv
+    cols = (0, h * dk, 2 * h * dk, 2 * h * dk + h * dv)
+    dev = "cuda"
+    S = torch.zeros((batch + 1, h, dk, dv), device=dev)
+    n = torch.zeros((batch + 1, h, dk), device=dev)
+    m = torch.zeros((batch + 1, h), device=dev)
+    weight = torch.ones(h * dv, device=dev)
+
+    def run(lens):
+        tokens = sum(lens)
+        packed = (torch.randn(tokens, width, device=dev) * 0.5).bfloat16()
+        pre = torch.randn(tokens, 2 * h, device=dev)
+        out = torch.empty((tokens, h * dv), dtype=torch.bfloat16, device=dev)
+        cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=dev)
+        ctx = types.SimpleNamespace(num_seqs=len(lens), h_seq_lens=lens, h_seq_slots=list(range(len(lens))),
+                                    cu_seqlens=cu, seq_slots=torch.arange(len(lens), dtype=torch.int32, device=dev))
+
+        def call():
+            ops.mlstm(packed, cols, pre, None, weight, out, ctx, S, n, m, h, dk, dv, 15.0, 1e-6)
+
+        for _ in range(3):
+            call()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(10):
+            call()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / 10
+
+    sec_p = run([prompt_len])
+    # per token and head: S^T q and the update k v^T over dk x (dv + 1), and the chunk's own
+    # scores and their products with the values at chunks of 64
+    flops = prompt_len * h * (4.0 * dk * (dv + 1) + 2.0 * 64 * (dk + dv + 1))
+    sec_d = run([1] * batch)
+    state_bytes = 2.0 * batch * h * dk * (dv + 1) * 4
+    return {
+        "recurrence_prefill_us": round(sec_p * 1e6, 1),
+        "recurrence_prefill_frac_fp32_matrix": round(flops / sec_p / (PEAK_TFLOPS["float32"] * 1e12), 4),
+        "recurrence_decode_us": round(sec_d * 1e6, 1),
+        "recurrence_decode_frac_hbm": round(state_bytes / sec_d / 1e9 / HBM_GBPS, 4),
+    }
+
+
+def run_design(args) -> int:
+    if args.design != "fokulorn":
+        print(f"unknown design {args.design!r}; known: fokulorn")
+        return 2
+    prompt_len = args.prompt_len or 2048
+    out = {"design": "Fokulorn", "beside": "Qwen3 of equal width, depth, heads and feed-forward width",
+           "dtype": "bf16", "data": "synthetic (uniform random token ids, random N(0,0.02) weights)",
+           "prompt_len": prompt_len, "batch": args.batch, "sizes": {}}
+    for name in [x for x in args.design_size.split(",") if x]:
+        z = DESIGN_SIZES[name]
+        row = {"config": z}
+        row["fokulorn"] = _time_model(fokulorn_body(z), prompt_len, args.batch, args.point_steps, prompt_len + 512)
+        print(f"[bench] {name} fokulorn {row['fokulorn']}", file=sys.stderr, flush=True)
+        row["qwen3"] = _time_model(qwen3_body(z), prompt_len, args.batch, args.point_steps, prompt_len + 512)
+        print(f"[bench] {name} qwen3 {row['qwen3']}", file=sys.stderr, flush=True)
+        row["kernels"] = _time_kernels(z, prompt_len, args.batch)
+        print(f"[bench] {name} kernels {row['kernels']}", file=sys.stderr, flush=True)
+        out["sizes"][name] = row
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -298,9 +462,14 @@ def main() -> int:
     ap.add_argument("--no-workloads", action="store_true", help="skip the scheduler workloads (processes of their own)")
     ap.add_argument("--peaks", action="store_true",
                     help="measure what the device reaches with library kernels (a large read, copy and square products) and exit")
+    ap.add_argument("--design", default=None,
+                    help="measure another architecture of the engine beside Qwen3 at equal size (fokulorn) and exit")
+    ap.add_argument("--design-size", default="2b,8b", help=f"sizes for --design: {', '.join(DESIGN_SIZES)}")
     args = ap.parse_args()
     if args.peaks:
         return measured_peaks()
+    if args.design is not None:
+        return run_design(args)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
         return 2
