@@ -1316,6 +1316,27 @@ def decode_attention_fused(
 # matrix-memory recurrence
 # --------------------------------------------------------------------------- #
 MLSTM_MAX_KEY_DIM = 256  # the scan stages a token's query and key of one head in LDS
+MLSTM_CHUNK = 64  # tokens a chunk of the chunked form
+MLSTM_CHUNKED_FROM = 16  # a step whose longest portion has so many tokens runs the chunked form
+
+
+def _mlstm_chunks(ctx):
+    """The step's chunk tables, made once a step and shared by its layers: per chunk
+    (request, first token, tokens, 0), per request (first chunk, chunks)."""
+    key = "mlstm_chunks"
+    found = ctx.extra.get(key) if hasattr(ctx, "extra") else None
+    if found is None:
+        chunks, per_seq, at = [], [], 0
+        for i, n in enumerate(ctx.h_seq_lens):
+            per_seq += [len(chunks) // 4, -(-n // MLSTM_CHUNK)]
+            for lo in range(0, n, MLSTM_CHUNK):
+                chunks += [i, at + lo, min(MLSTM_CHUNK, n - lo), 0]
+            at += n
+        dev = ctx.seq_slots.device
+        found = (upload_ints(chunks, dev), len(chunks) // 4, upload_ints(per_seq, dev))
+        if hasattr(ctx, "extra"):
+            ctx.extra[key] = found
+    return found
 
 
 def mlstm(
@@ -1334,6 +1355,7 @@ def mlstm(
     dv: int,
     cap: float,
     eps: float,
+    chunked: Optional[bool] = None,
 ) -> None:
     """The matrix-memory mixer between its projections and its output projection.
 
@@ -1344,7 +1366,11 @@ def mlstm(
     dk, dv]``, ``n [slots, heads, dk]``, ``m [slots, heads]`` (float32) is read at the rows
     ``ctx.seq_slots`` and left as it is after each request's last token of the step.
     ``out [T, heads * dv]``: every head's output divided by its root mean square, times
-    ``norm_weight``, times the sigmoid of the output gate."""
+    ``norm_weight``, times the sigmoid of the output gate.
+
+    Two forms of the recurrence: token by token (steps of single tokens and short portions),
+    and in chunks of 64 tokens on the matrix cores (``chunked``; by default a step whose
+    longest portion has 16 tokens or more).  They differ by rounding."""
     tokens, width = packed.shape
     q_col, k_col, v_col, g_col = (int(c) for c in columns)
     _need(packed, "packed projections")
@@ -1382,14 +1408,30 @@ def mlstm(
         ),
         "rl_mlstm_gates",
     )
-    _ok(
-        lib.rl_mlstm_scan(
-            _p(packed), width, q_col, k_col, v_col, _p(log_keep), _p(log_take), _p(ctx.cu_seqlens),
-            _p(ctx.seq_slots), _p(S), _p(n), _p(raw), ctx.num_seqs, heads, dk, dv,
-            ctypes.c_float(float(dk) ** -0.5), _tag(packed.dtype), _stream(),
-        ),
-        "rl_mlstm_scan",
-    )
+    chunked = max(ctx.h_seq_lens, default=0) >= MLSTM_CHUNKED_FROM if chunked is None else chunked
+    if chunked:
+        # portions of prompts: every chunk of 64 tokens at once on the matrix cores
+        chunks, nchunks, seq_chunks = _mlstm_chunks(ctx)
+        U = torch.empty((nchunks, heads, dk, dv), dtype=torch.float32, device=dev)
+        Un = torch.empty((nchunks, heads, dk), dtype=torch.float32, device=dev)
+        decay = torch.empty((nchunks, heads), dtype=torch.float32, device=dev)
+        _ok(
+            lib.rl_mlstm_chunked(
+                _p(packed), width, q_col, k_col, v_col, _p(log_keep), _p(log_take), _p(chunks), nchunks,
+                _p(seq_chunks), _p(ctx.seq_slots), ctx.num_seqs, _p(U), _p(Un), _p(decay), _p(S), _p(n), _p(raw),
+                heads, dk, dv, ctypes.c_float(float(dk) ** -0.5), _tag(packed.dtype), _stream(),
+            ),
+            "rl_mlstm_chunked",
+        )
+    else:
+        _ok(
+            lib.rl_mlstm_scan(
+                _p(packed), width, q_col, k_col, v_col, _p(log_keep), _p(log_take), _p(ctx.cu_seqlens),
+                _p(ctx.seq_slots), _p(S), _p(n), _p(raw), ctx.num_seqs, heads, dk, dv,
+                ctypes.c_float(float(dk) ** -0.5), _tag(packed.dtype), _stream(),
+            ),
+            "rl_mlstm_scan",
+        )
     _ok(
         lib.rl_mlstm_finish(
             _p(raw), _p(m_tok), _p(packed), width, g_col, _p(norm_weight), _p(out), tokens, heads, dv,

@@ -78,14 +78,17 @@ def _mlstm_reference(q, k, v, g, pre_i, pre_f, cap, weight, eps, state=None):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("chunked", [False, True, None])
 @pytest.mark.parametrize("heads,dk,dv", [(3, 16, 40), (1, 8, 8), (2, 80, 72), (2, 256, 20), (5, 33, 7), (2, 128, 130)])
-def test_recurrence_kernels_against_plain(dtype, heads, dk, dv):
+def test_recurrence_kernels_against_plain(dtype, heads, dk, dv, chunked):
     """Three requests of unequal length in one launch, in slots that are not in order, each cut
-    into two steps at another place; the state between the steps is the kernels' own."""
+    into two steps at another place; the state between the steps is the kernels' own.  Token
+    by token, in chunks of 64 (a request of 200 tokens crosses three chunk edges, one ends at
+    an edge), and as the step's shape decides."""
     from rapid_llm_amd.kernels import ops
 
     torch.manual_seed(heads * 1000 + dk + dv)
-    lens, slots, cuts = [37, 1, 70], [4, 0, 2], [2, 1, 33]
+    lens, slots, cuts = [37, 1, 200, 128], [4, 0, 2, 5], [2, 1, 33, 64]
     cap, eps = 9.0, 1e-5
     qk, vv = heads * dk, heads * dv
     width = 2 * qk + 2 * vv
@@ -113,7 +116,7 @@ def test_recurrence_kernels_against_plain(dtype, heads, dk, dv):
         out = torch.empty((packed.shape[0], vv), dtype=dtype, device=DEV)
         ctx = _ctx([spans[i][1] - spans[i][0] for i in live], [slots[i] for i in live])
         ops.mlstm(packed, cols, pre, bias.to(DEV), weight.to(DEV), out, ctx, S, n_state, m_state,
-                  heads, dk, dv, cap, eps)
+                  heads, dk, dv, cap, eps, chunked=chunked)
         at = 0
         for i in live:
             n = spans[i][1] - spans[i][0]
