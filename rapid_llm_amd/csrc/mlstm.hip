@@ -16,8 +16,8 @@
 // Three kernels a step:
 //   gates   one wave per (request, head): i, f, the maxima m_t, and per token the logarithms
 //           of the two decay factors (log keep = f_t + m_{t-1} - m_t, log take = i_t - m_t,
-//           both <= 0).  Activations of 64 tokens are computed side by side, the max-plus
-//           recurrence walks them in order.
+//           both <= 0 up to rounding).  Activations side by side, the max-plus recurrence
+//           as a scan over the workgroup.
 //   scan    per (request, head, block of columns): the state update and S^T q token by token,
 //           the tokens' rows staged through LDS sixteen at a time.
 //   finish  per (token, head): the division, the head's unit root mean square, the weight over
@@ -34,37 +34,54 @@ __device__ inline float soft_cap(float x, float cap) { return cap * tanhf(x / ca
 __device__ inline float log_sigmoid(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
 // gate_pre [tokens, 2 * heads]: the input gates' pre-activations, then the forget gates'.
-__global__ __launch_bounds__(RL_WAVE) void mlstm_gates_kernel(
+// A token maps the maximum m to max(m + f, i).  Two tokens in a row map it to
+// max(m + f1 + f2, max(i1 + f2, i2)): such pairs (F, G) are folded over a wave by an inclusive
+// scan, the waves' totals over the workgroup through LDS, and every lane applies its pair to
+// the maximum that entered.  A workgroup of W waves takes 64 W tokens at a time.
+__global__ __launch_bounds__(1024) void mlstm_gates_kernel(
     const float* __restrict__ gate_pre, const float* __restrict__ gate_bias,
     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, float* __restrict__ m_state,
     float* __restrict__ log_keep, float* __restrict__ log_take, float* __restrict__ m_tok, int heads,
     float cap) {
-    const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    __shared__ float wF[16], wG[16];
+    const int s = blockIdx.x, h = blockIdx.y;
+    const int lane = threadIdx.x & (RL_WAVE - 1), wave = threadIdx.x / RL_WAVE;
+    const int waves = blockDim.x / RL_WAVE;
     const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
     const int slot = seq_slots[s];
-    float m = m_state[(size_t)slot * heads + h];
+    float m = m_state[(size_t)slot * heads + h];  // the maximum that enters this round
     const float bi = gate_bias ? gate_bias[h] : 0.f;
     const float bf = gate_bias ? gate_bias[heads + h] : 0.f;
-    for (int base = t0; base < t1; base += RL_WAVE) {
-        const int t = base + lane;
+    for (int base = t0; base < t1; base += blockDim.x) {
+        const int t = base + threadIdx.x;
         const bool valid = t < t1;
         float gi = 0.f, gf = 0.f;
         if (valid) {
             gi = soft_cap(gate_pre[(size_t)t * 2 * heads + h] + bi, cap);
             gf = log_sigmoid(soft_cap(gate_pre[(size_t)t * 2 * heads + heads + h] + bf, cap));
         }
-        const int count = min(RL_WAVE, t1 - base);
-        float before = 0.f, mine = 0.f;
-        for (int u = 0; u < count; ++u) {
-            const float fu = __shfl(gf, u, RL_WAVE);
-            const float iu = __shfl(gi, u, RL_WAVE);
-            const float m_new = fmaxf(fu + m, iu);
-            if (lane == u) {
-                before = m;
-                mine = m_new;
+        float F = valid ? gf : 0.f, G = valid ? gi : -INFINITY;
+#pragma unroll
+        for (int off = 1; off < RL_WAVE; off <<= 1) {
+            const float Fu = __shfl_up(F, off, RL_WAVE);
+            const float Gu = __shfl_up(G, off, RL_WAVE);
+            if (lane >= off) {
+                G = fmaxf(Gu + F, G);
+                F = Fu + F;
             }
-            m = m_new;
         }
+        __syncthreads();  // the last round's totals are read
+        if (lane == RL_WAVE - 1) {
+            wF[wave] = F;
+            wG[wave] = G;
+        }
+        __syncthreads();
+        float m_in = m;  // what enters this wave's 64 tokens
+        for (int w = 0; w < wave; ++w) m_in = fmaxf(m_in + wF[w], wG[w]);
+        const float mine = fmaxf(m_in + F, G);
+        const float up = __shfl_up(mine, 1, RL_WAVE);
+        const float before = lane == 0 ? m_in : up;
+        for (int w = 0; w < waves; ++w) m = fmaxf(m + wF[w], wG[w]);
         if (valid) {
             const size_t at = (size_t)t * heads + h;
             log_keep[at] = gf + before - mine;
@@ -72,7 +89,7 @@ __global__ __launch_bounds__(RL_WAVE) void mlstm_gates_kernel(
             m_tok[at] = mine;
         }
     }
-    if (lane == 0) m_state[(size_t)slot * heads + h] = m;
+    if (threadIdx.x == 0) m_state[(size_t)slot * heads + h] = m;
 }
 
 // One wave per (request, head, block of columns).  A wave's 64 lanes are `slices` groups of
@@ -154,6 +171,63 @@ __global__ __launch_bounds__(RL_WAVE) void mlstm_scan_kernel(
     }
 }
 
+// A step of single tokens: the state is read, updated and written back once, as a stream.
+// One workgroup per (token, head, 64 columns): lane = column (64 consecutive floats of a state
+// row are one 256-byte access), the four waves split the rows and their sums meet in LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void mlstm_step_kernel(
+    const T* __restrict__ packed, int row_width, int q_col, int k_col, int v_col,
+    const float* __restrict__ log_keep, const float* __restrict__ log_take,
+    const int* __restrict__ seq_slots, float* __restrict__ S_state, float* __restrict__ n_state,
+    float* __restrict__ raw, int heads, int dk, int dv, float q_scale) {
+    __shared__ float sq[256], sk[256];
+    __shared__ float part[4][RL_WAVE];
+    const int t = blockIdx.x, h = blockIdx.y;
+    const int lane = threadIdx.x & (RL_WAVE - 1), wave = threadIdx.x / RL_WAVE;
+    const int j = blockIdx.z * RL_WAVE + lane;
+    const int slot = seq_slots[t];
+    const T* row = packed + (size_t)t * row_width;
+    if ((int)threadIdx.x < dk) {
+        sq[threadIdx.x] = to_float(row[q_col + (size_t)h * dk + threadIdx.x]);
+        sk[threadIdx.x] = to_float(row[k_col + (size_t)h * dk + threadIdx.x]);
+    }
+    const float keep = expf(log_keep[(size_t)t * heads + h]);
+    const float take = expf(log_take[(size_t)t * heads + h]);
+    __syncthreads();
+    const bool live = j <= dv, is_n = j == dv;
+    const float tv = take * (is_n ? 1.f : (j < dv ? to_float(row[v_col + (size_t)h * dv + j]) : 0.f));
+    float* column = is_n ? n_state + ((size_t)slot * heads + h) * dk
+                         : S_state + ((size_t)slot * heads + h) * dk * dv + j;
+    const size_t stride = is_n ? 1 : dv;
+    const int per = (dk + 3) / 4;
+    const int d_lo = wave * per, d_hi = min(dk, d_lo + per);
+    float acc = 0.f;
+    if (live) {
+        int d = d_lo;
+        for (; d + 8 <= d_hi; d += 8) {
+            float s[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s[u] = column[(size_t)(d + u) * stride];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                s[u] = keep * s[u] + tv * sk[d + u];
+                acc += s[u] * sq[d + u];
+                column[(size_t)(d + u) * stride] = s[u];
+            }
+        }
+        for (; d < d_hi; ++d) {
+            const float v = keep * column[(size_t)d * stride] + tv * sk[d];
+            acc += v * sq[d];
+            column[(size_t)d * stride] = v;
+        }
+    }
+    part[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && live)
+        raw[((size_t)t * heads + h) * (dv + 1) + j] =
+            (part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane]) * q_scale;
+}
+
 // out[t, h * dv + j] = o_j / rms(o) * weight[h * dv + j] * sigmoid(gate[t, h * dv + j]) with
 // o = raw[.., :dv] / (max(|raw[.., dv]|, exp(-m_t)) + 1e-6).  One wave per (token, head).
 template <typename T>
@@ -229,7 +303,8 @@ __device__ inline void chunk_gates(const float* __restrict__ log_keep, const flo
 }
 
 // U[c][h][d][j] = sum_s w_s k_s[d] v_s[j], Un[c][h][d] = sum_s w_s k_s[d], decay[c][h] = A_last.
-// Wave w owns the rows d of the tiles w, w + 4, ... (RT of them), and all MC_CT column tiles.
+// Wave w owns the column tiles 2 w and 2 w + 1 and all RT row tiles of 16 state rows: a value
+// is loaded by one wave only and meets every key row of the slab.
 template <typename T, int RT>
 __global__ __launch_bounds__(256) void mlstm_chunk_state_kernel(
     const T* __restrict__ packed, int row_width, int k_col, int v_col, const float* __restrict__ log_keep,
@@ -246,22 +321,35 @@ __global__ __launch_bounds__(256) void mlstm_chunk_state_kernel(
     const float a_last = sA[count - 1];
     if (threadIdx.x < MC_L) sW[threadIdx.x] = threadIdx.x < count ? expf(a_last - sA[threadIdx.x] + sB[threadIdx.x]) : 0.f;
     if (threadIdx.x == 0 && blockIdx.z == 0) decay[(size_t)c * heads + h] = a_last;
-    f32x4 acc[RT][MC_CT];
+    f32x4 acc[RT][2];
 #pragma unroll
     for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int ct = 0; ct < MC_CT; ++ct) acc[i][ct] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int ct = 0; ct < 2; ++ct) acc[i][ct] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float un = 0.f;
+    // thread d holds channel d of the keys of a slab's 16 tokens: sixteen loads asked for at
+    // once, the next slab's while this one is multiplied
+    // (no load stands behind a condition: addresses are clamped into the chunk and what lies
+    // beyond it is dropped afterwards, so that the loads of a batch travel together)
+    const int kd = threadIdx.x;
+    const T* kcol = packed + (size_t)begin * row_width + k_col + (size_t)h * dk + min(kd, dk - 1);
+    float kv[16];
+    auto load_keys = [&](int base) {
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const float x = to_float(kcol[(size_t)min(base + u, count - 1) * row_width]);
+            kv[u] = (kd < dk && base + u < count) ? x : 0.f;
+        }
+    };
+    load_keys(0);
     for (int base = 0; base < count; base += 16) {
         __syncthreads();  // sW is written; the last slab is read
-        for (int idx = threadIdx.x; idx < 16 * dk16; idx += 256) {
-            const int u = idx / dk16, d = idx - u * dk16;
-            float v = 0.f;
-            if (base + u < count && d < dk)
-                v = sW[base + u] * to_float(packed[(size_t)(begin + base + u) * row_width + k_col + (size_t)h * dk + d]);
-            sK[u][d] = v;
+        if (kd < dk16) {
+#pragma unroll
+            for (int u = 0; u < 16; ++u) sK[u][kd] = sW[base + u] * kv[u];
         }
         __syncthreads();
+        if (base + 16 < count) load_keys(base + 16);
         if (blockIdx.z == 0 && (int)threadIdx.x < dk) {
 #pragma unroll
             for (int u = 0; u < 16; ++u) un += sK[u][threadIdx.x];
@@ -269,21 +357,21 @@ __global__ __launch_bounds__(256) void mlstm_chunk_state_kernel(
 #pragma unroll
         for (int kk = 0; kk < 16; kk += 4) {
             const int u = kk + g;
-            float a[RT];
+            const bool live = base + u < count;
+            const T* vrow = packed + (size_t)(begin + min(base + u, count - 1)) * row_width + v_col + (size_t)h * dv;
+            float b[2];
+#pragma unroll
+            for (int ct = 0; ct < 2; ++ct) {
+                const int j = j0 + 16 * (2 * wave + ct) + l16;
+                const float x = to_float(vrow[min(j, dv - 1)]);
+                b[ct] = (live && j < dv) ? x : 0.f;
+            }
 #pragma unroll
             for (int i = 0; i < RT; ++i) {
-                const int d0 = 16 * (wave + 4 * i);
-                a[i] = d0 < dk16 ? sK[u][d0 + l16] : 0.f;
-            }
-            const bool live = base + u < count;
-            const T* vrow = packed + (size_t)(begin + base + u) * row_width + v_col + (size_t)h * dv;
+                const float a = 16 * i < dk16 ? sK[u][16 * i + l16] : 0.f;
 #pragma unroll
-            for (int ct = 0; ct < MC_CT; ++ct) {
-                const int j = j0 + 16 * ct + l16;
-                const float b = (live && j < dv) ? to_float(vrow[j]) : 0.f;
-#pragma unroll
-                for (int i = 0; i < RT; ++i)
-                    acc[i][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b, acc[i][ct], 0, 0, 0);
+                for (int ct = 0; ct < 2; ++ct)
+                    acc[i][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ct], acc[i][ct], 0, 0, 0);
             }
         }
     }
@@ -291,10 +379,10 @@ __global__ __launch_bounds__(256) void mlstm_chunk_state_kernel(
 #pragma unroll
     for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int ct = 0; ct < MC_CT; ++ct)
+        for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int d = 16 * (wave + 4 * i) + 4 * g + r, j = j0 + 16 * ct + l16;
+                const int d = 16 * i + 4 * g + r, j = j0 + 16 * (2 * wave + ct) + l16;
                 if (d < dk && j < dv) out[(size_t)d * dv + j] = acc[i][ct][r];
             }
     if (blockIdx.z == 0 && (int)threadIdx.x < dk) Un[((size_t)c * heads + h) * dk + threadIdx.x] = un;
@@ -319,15 +407,15 @@ __global__ __launch_bounds__(256) void mlstm_chunk_carry_kernel(
     const size_t stride = is_n ? (size_t)heads * dk : (size_t)heads * per;
     float s = *state;
     int c = 0;
-    for (; c + 4 <= nc; c += 4) {
-        float u[4], f[4];
+    for (; c + 8 <= nc; c += 8) {
+        float u[8], f[8];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
+        for (int k = 0; k < 8; ++k) {
             u[k] = buf[(size_t)(c0 + c + k) * stride];
             f[k] = expf(decay[(size_t)(c0 + c + k) * heads + h]);
         }
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
+        for (int k = 0; k < 8; ++k) {
             buf[(size_t)(c0 + c + k) * stride] = s;
             s = f[k] * s + u[k];
         }
@@ -341,7 +429,9 @@ __global__ __launch_bounds__(256) void mlstm_chunk_carry_kernel(
 }
 
 // raw[t][h][j] = q_scale * (exp(A_t) S_in^T q_t + sum_{s<=t} w_ts (q_t . k_s) v_s)[j]; the entry
-// dv of a row is the same with n_in and the value 1.  Wave w owns the rows 16 w .. 16 w + 15.
+// dv of a row is the same with n_in and the value 1.  For the scores wave w owns the rows
+// 16 w .. 16 w + 15; for the products with values and state it owns the column tiles 2 w and
+// 2 w + 1 of all 64 rows, so that a value or a state element is loaded by one wave only.
 template <typename T>
 __global__ __launch_bounds__(256) void mlstm_chunk_output_kernel(
     const T* __restrict__ packed, int row_width, int q_col, int k_col, int v_col,
@@ -363,29 +453,45 @@ __global__ __launch_bounds__(256) void mlstm_chunk_output_kernel(
     if (threadIdx.x < MC_L) sE[threadIdx.x] = expf(sA[threadIdx.x]);
     if (first && (int)threadIdx.x < dk) sN[threadIdx.x] = Un[((size_t)c * heads + h) * dk + threadIdx.x];
 
-    auto stage = [&](int d0, bool keys) {
-        for (int idx = threadIdx.x; idx < MC_L * MC_SLAB; idx += 256) {
-            const int t = idx / MC_SLAB, dd = idx - t * MC_SLAB;
-            float q = 0.f, k = 0.f;
-            if (t < count && d0 + dd < dk) {
-                const T* row = packed + (size_t)(begin + t) * row_width + (size_t)h * dk + d0 + dd;
-                q = to_float(row[q_col]);
-                if (keys) k = to_float(row[k_col]);
+    // thread (t0, dd) holds channel d0 + dd of the tokens t0, t0 + 8, ...: eight (or sixteen)
+    // loads asked for at once
+    const int sdd = threadIdx.x % MC_SLAB, st0 = threadIdx.x / MC_SLAB;
+    float gq[8], gk[8];
+    auto stage_load = [&](int d0, bool keys) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int t = st0 + 8 * i;
+            const bool live = t < count && d0 + sdd < dk;
+            const T* row = packed + (size_t)(begin + min(t, count - 1)) * row_width + (size_t)h * dk +
+                           min(d0 + sdd, dk - 1);
+            const float xq = to_float(row[q_col]);
+            gq[i] = live ? xq : 0.f;
+            if (keys) {
+                const float xk = to_float(row[k_col]);
+                gk[i] = live ? xk : 0.f;
             }
-            sQ[t][dd] = q;
-            if (keys) sK[t][dd] = k;
+        }
+    };
+    auto stage_store = [&](bool keys) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            sQ[st0 + 8 * i][sdd] = gq[i];
+            if (keys) sK[st0 + 8 * i][sdd] = gk[i];
         }
     };
 
+    const int jw = j0 + 32 * wave + l16;  // this lane's column of the wave's first tile
     // ---- scores of the chunk's own tokens
     f32x4 p[4];
 #pragma unroll
     for (int ct = 0; ct < 4; ++ct) p[ct] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float dot = 0.f;  // q_t . n_in, by the thread of row t
+    stage_load(0, true);
     for (int d0 = 0; d0 < dk4; d0 += MC_SLAB) {
         __syncthreads();
-        stage(d0, true);
+        stage_store(true);
         __syncthreads();
+        if (d0 + MC_SLAB < dk4) stage_load(d0 + MC_SLAB, true);  // the next slab travels meanwhile
         if (first && threadIdx.x < MC_L) {
             for (int dd = 0; dd < MC_SLAB && d0 + dd < dk; ++dd) dot += sQ[threadIdx.x][dd] * sN[d0 + dd];
         }
@@ -397,6 +503,20 @@ __global__ __launch_bounds__(256) void mlstm_chunk_output_kernel(
                 p[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, sK[16 * ct + l16][kk + g], p[ct], 0, 0, 0);
         }
     }
+    // the chunk's values of this wave's two column tiles and the first slab of the queries
+    // again, asked for while the weights are made
+    float bv[MC_L / 4][2];
+#pragma unroll
+    for (int kq = 0; kq < MC_L / 4; ++kq) {
+        const int u = 4 * kq + g;
+        const T* vrow = packed + (size_t)(begin + min(u, count - 1)) * row_width + v_col + (size_t)h * dv;
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) {
+            const float x = to_float(vrow[min(jw + 16 * ct, dv - 1)]);
+            bv[kq][ct] = (u < count && jw + 16 * ct < dv) ? x : 0.f;
+        }
+    }
+    stage_load(0, false);
     // ---- decay weights, the causal mask, row sums (the normaliser's column)
     float rs[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -417,46 +537,72 @@ __global__ __launch_bounds__(256) void mlstm_chunk_output_kernel(
     if (first && threadIdx.x < MC_L) sDot[threadIdx.x] = dot;
     __syncthreads();
     // ---- weights times values
-    f32x4 acc[MC_CT];
+    f32x4 acc[4][2];
 #pragma unroll
-    for (int ct = 0; ct < MC_CT; ++ct) acc[ct] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    for (int kk = 0; kk < count; kk += 4) {
-        const float a = sP[16 * wave + l16][kk + g];
-        const bool live = kk + g < count;
-        const T* vrow = packed + (size_t)(begin + kk + g) * row_width + v_col + (size_t)h * dv;
+    for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
-        for (int ct = 0; ct < MC_CT; ++ct) {
-            const int j = j0 + 16 * ct + l16;
-            const float b = (live && j < dv) ? to_float(vrow[j]) : 0.f;
-            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[ct], 0, 0, 0);
+        for (int ct = 0; ct < 2; ++ct) acc[rt][ct] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kq = 0; kq < MC_L / 4; ++kq) {
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+            const float a = sP[16 * rt + l16][4 * kq + g];
+#pragma unroll
+            for (int ct = 0; ct < 2; ++ct)
+                acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bv[kq][ct], acc[rt][ct], 0, 0, 0);
         }
     }
     // ---- the entering state: rows of q times exp(A_t)
     const float* Sin = U + ((size_t)c * heads + h) * dk * dv;
-    const float e_row = sE[16 * wave + l16];
+    float e_row[4];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) e_row[rt] = sE[16 * rt + l16];
+    float bs[MC_SLAB / 4][2];  // a slab's rows of the entering state, asked for a slab ahead
+    auto load_state = [&](int d0) {
+#pragma unroll
+        for (int kq = 0; kq < MC_SLAB / 4; ++kq) {
+            const int d = d0 + 4 * kq + g;
+#pragma unroll
+            for (int ct = 0; ct < 2; ++ct) {
+                const float x = Sin[(size_t)min(d, dk - 1) * dv + min(jw + 16 * ct, dv - 1)];
+                bs[kq][ct] = (d < dk && jw + 16 * ct < dv) ? x : 0.f;
+            }
+        }
+    };
+    load_state(0);
     for (int d0 = 0; d0 < dk4; d0 += MC_SLAB) {
         __syncthreads();
-        stage(d0, false);
+        stage_store(false);
         __syncthreads();
+        if (d0 + MC_SLAB < dk4) stage_load(d0 + MC_SLAB, false);
+        float b[MC_SLAB / 4][2];
 #pragma unroll
-        for (int kk = 0; kk < MC_SLAB; kk += 4) {
-            const int d = d0 + kk + g;
-            const float a = sQ[16 * wave + l16][kk + g] * e_row;
+        for (int kq = 0; kq < MC_SLAB / 4; ++kq) {
+            b[kq][0] = bs[kq][0];
+            b[kq][1] = bs[kq][1];
+        }
+        if (d0 + MC_SLAB < dk4) load_state(d0 + MC_SLAB);
 #pragma unroll
-            for (int ct = 0; ct < MC_CT; ++ct) {
-                const int j = j0 + 16 * ct + l16;
-                const float b = (d < dk && j < dv) ? Sin[(size_t)d * dv + j] : 0.f;
-                acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[ct], 0, 0, 0);
+        for (int kq = 0; kq < MC_SLAB / 4; ++kq) {
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                const float a = sQ[16 * rt + l16][4 * kq + g] * e_row[rt];
+#pragma unroll
+                for (int ct = 0; ct < 2; ++ct)
+                    acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[kq][ct], acc[rt][ct], 0, 0, 0);
             }
         }
     }
 #pragma unroll
-    for (int ct = 0; ct < MC_CT; ++ct)
+    for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int t = 16 * wave + 4 * g + r, j = j0 + 16 * ct + l16;
-            if (t < count && j < dv) raw[((size_t)(begin + t) * heads + h) * (dv + 1) + j] = acc[ct][r] * q_scale;
-        }
+        for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = 16 * rt + 4 * g + r, j = jw + 16 * ct;
+                if (t < count && j < dv)
+                    raw[((size_t)(begin + t) * heads + h) * (dv + 1) + j] = acc[rt][ct][r] * q_scale;
+            }
     if (first && (int)threadIdx.x < count) {
         const int t = threadIdx.x;
         raw[((size_t)(begin + t) * heads + h) * (dv + 1) + dv] = (sRow[t] + sE[t] * sDot[t]) * q_scale;
@@ -474,10 +620,14 @@ static int mlstm_slices(int dk) {
 
 extern "C" int rl_mlstm_gates(const float* gate_pre, const float* gate_bias, const int* cu_seqlens,
                               const int* seq_slots, float* m_state, float* log_keep, float* log_take,
-                              float* m_tok, int num_seqs, int heads, float cap, hipStream_t stream) {
+                              float* m_tok, int num_seqs, int heads, float cap, int longest,
+                              hipStream_t stream) {
     if (num_seqs <= 0) return RL_OK;
     if (heads < 1 || heads > 65535 || !(cap > 0.f)) return RL_ERR_ARG;
-    hipLaunchKernelGGL(mlstm_gates_kernel, dim3(num_seqs, heads), dim3(RL_WAVE), 0, stream, gate_pre,
+    // as many waves as the longest request of the step has blocks of 64 tokens, up to 16
+    int waves = (longest + RL_WAVE - 1) / RL_WAVE;
+    waves = waves < 1 ? 1 : (waves > 16 ? 16 : waves);
+    hipLaunchKernelGGL(mlstm_gates_kernel, dim3(num_seqs, heads), dim3(waves * RL_WAVE), 0, stream, gate_pre,
                        gate_bias, cu_seqlens, seq_slots, m_state, log_keep, log_take, m_tok, heads, cap);
     return rl_launch_status();
 }
@@ -543,18 +693,20 @@ extern "C" int rl_mlstm_chunked(const void* packed, int row_width, int q_col, in
         return RL_ERR_ARG;
     const int jblocks = (dv + MC_JB - 1) / MC_JB;
     if (jblocks > 65535) return RL_ERR_ARG;
-    const int row_tiles = ((dk + 15) / 16 + 3) / 4;  // tiles of 16 state rows a wave
+    const int row_tiles = (dk + 15) / 16;  // tiles of 16 state rows
     dim3 grid(nchunks, heads, jblocks), block(256);
 #define ML_STATE(TT, RTV)                                                                                      \
     hipLaunchKernelGGL((mlstm_chunk_state_kernel<TT, RTV>), grid, block, 0, stream, (const TT*)packed, row_width, \
                        k_col, v_col, log_keep, log_take, chunks, U, Un, decay, heads, dk, dv)
 #define ML_STATE_T(TT)          \
-    if (row_tiles <= 1)         \
-        ML_STATE(TT, 1);        \
-    else if (row_tiles == 2)    \
+    if (row_tiles <= 2)         \
         ML_STATE(TT, 2);        \
+    else if (row_tiles <= 4)    \
+        ML_STATE(TT, 4);        \
+    else if (row_tiles <= 8)    \
+        ML_STATE(TT, 8);        \
     else                        \
-        ML_STATE(TT, 4)
+        ML_STATE(TT, 16)
     if (act_type == RL_F32) {
         ML_STATE_T(float);
     } else if (act_type == RL_BF16) {
@@ -574,5 +726,31 @@ extern "C" int rl_mlstm_chunked(const void* packed, int row_width, int q_col, in
         hipLaunchKernelGGL(mlstm_chunk_output_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)packed,
                            row_width, q_col, k_col, v_col, log_keep, log_take, chunks, U, Un, raw, heads, dk, dv,
                            q_scale);
+    return rl_launch_status();
+}
+
+// rl_mlstm_scan for a step in which every request brings one token (request i = token i).
+extern "C" int rl_mlstm_step(const void* packed, int row_width, int q_col, int k_col, int v_col,
+                             const float* log_keep, const float* log_take, const int* seq_slots,
+                             float* S_state, float* n_state, float* raw, int tokens, int heads, int dk,
+                             int dv, float q_scale, int act_type, hipStream_t stream) {
+    if (tokens <= 0) return RL_OK;
+    if (heads < 1 || heads > 65535 || dk < 1 || dk > 256 || dv < 1) return RL_ERR_ARG;
+    if (q_col < 0 || k_col < 0 || v_col < 0 || q_col + heads * dk > row_width ||
+        k_col + heads * dk > row_width || v_col + heads * dv > row_width)
+        return RL_ERR_ARG;
+    const int blocks = (dv + 1 + RL_WAVE - 1) / RL_WAVE;
+    if (blocks > 65535) return RL_ERR_ARG;
+    dim3 grid(tokens, heads, blocks), block(256);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(mlstm_step_kernel<float>, grid, block, 0, stream, (const float*)packed, row_width,
+                           q_col, k_col, v_col, log_keep, log_take, seq_slots, S_state, n_state, raw, heads, dk,
+                           dv, q_scale);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(mlstm_step_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)packed, row_width,
+                           q_col, k_col, v_col, log_keep, log_take, seq_slots, S_state, n_state, raw, heads, dk,
+                           dv, q_scale);
+    else
+        return RL_ERR_ARG;
     return rl_launch_status();
 }

@@ -1368,9 +1368,10 @@ def mlstm(
     ``out [T, heads * dv]``: every head's output divided by its root mean square, times
     ``norm_weight``, times the sigmoid of the output gate.
 
-    Two forms of the recurrence: token by token (steps of single tokens and short portions),
-    and in chunks of 64 tokens on the matrix cores (``chunked``; by default a step whose
-    longest portion has 16 tokens or more).  They differ by rounding."""
+    Three forms of the recurrence, which differ by rounding: a step of single tokens streams
+    every state through once; short portions run token by token with the state in registers;
+    and ``chunked`` (by default a step whose longest portion has 16 tokens or more) runs chunks
+    of 64 tokens on the matrix cores."""
     tokens, width = packed.shape
     q_col, k_col, v_col, g_col = (int(c) for c in columns)
     _need(packed, "packed projections")
@@ -1404,7 +1405,8 @@ def mlstm(
     _ok(
         lib.rl_mlstm_gates(
             _p(gate_pre), _p(gate_bias), _p(ctx.cu_seqlens), _p(ctx.seq_slots), _p(m), _p(log_keep),
-            _p(log_take), _p(m_tok), ctx.num_seqs, heads, ctypes.c_float(cap), _stream(),
+            _p(log_take), _p(m_tok), ctx.num_seqs, heads, ctypes.c_float(cap), max(ctx.h_seq_lens, default=1),
+            _stream(),
         ),
         "rl_mlstm_gates",
     )
@@ -1422,6 +1424,16 @@ def mlstm(
                 heads, dk, dv, ctypes.c_float(float(dk) ** -0.5), _tag(packed.dtype), _stream(),
             ),
             "rl_mlstm_chunked",
+        )
+    elif tokens == ctx.num_seqs:
+        # single tokens only: the state goes through once, as a stream
+        _ok(
+            lib.rl_mlstm_step(
+                _p(packed), width, q_col, k_col, v_col, _p(log_keep), _p(log_take), _p(ctx.seq_slots), _p(S),
+                _p(n), _p(raw), tokens, heads, dk, dv, ctypes.c_float(float(dk) ** -0.5), _tag(packed.dtype),
+                _stream(),
+            ),
+            "rl_mlstm_step",
         )
     else:
         _ok(

@@ -82,7 +82,7 @@ def _mlstm_reference(q, k, v, g, pre_i, pre_f, cap, weight, eps, state=None):
 @pytest.mark.parametrize("heads,dk,dv", [(3, 16, 40), (1, 8, 8), (2, 80, 72), (2, 256, 20), (5, 33, 7), (2, 128, 130)])
 def test_recurrence_kernels_against_plain(dtype, heads, dk, dv, chunked):
     """Three requests of unequal length in one launch, in slots that are not in order, each cut
-    into two steps at another place; the state between the steps is the kernels' own.  Token
+    into three steps, the last of one token; the state between the steps is the kernels' own.  Token
     by token, in chunks of 64 (a request of 200 tokens crosses three chunk edges, one ends at
     an edge), and as the step's shape decides."""
     from rapid_llm_amd.kernels import ops
@@ -108,8 +108,8 @@ def test_recurrence_kernels_against_plain(dtype, heads, dk, dv, chunked):
     for s in slots:  # a slot that is taken starts at zero; the others hold what must never be read
         S[s], n_state[s], m_state[s] = 0, 0, 0
     got = [[] for _ in lens]
-    for part in range(2):
-        spans = [(0, c) if part == 0 else (c, n) for c, n in zip(cuts, lens)]
+    for part in range(3):  # the last step brings the last token of every longer request alone
+        spans = [((0, c), (c, max(c, n - 1)), (max(c, n - 1), n))[part] for c, n in zip(cuts, lens)]
         live = [i for i, (a, b) in enumerate(spans) if b > a]
         packed = torch.cat([reqs[i][0][spans[i][0]:spans[i][1]] for i in live]).to(DEV)
         pre = torch.cat([reqs[i][1][spans[i][0]:spans[i][1]] for i in live]).to(DEV)
