@@ -44,8 +44,8 @@ class AttentionMixerConfig:
             raise ConfigError(f"{where}: the values are the keys, so vdim {vdim!r} must equal dim {dim}")
         if heads % kv_heads:
             raise ConfigError(f"{where}: {heads} heads are not divisible by {kv_heads} kv_heads")
-        if dim % 8 or dim > 256:
-            raise ConfigError(f"{where}: the attention kernels take head sizes in steps of 8 up to 256, got {dim}")
+        if dim % 2 or dim > 256:
+            raise ConfigError(f"{where}: the attention kernels take even head sizes up to 256, got {dim}")
         mask = data.get("mask")
         window = 0
         if mask is not None:

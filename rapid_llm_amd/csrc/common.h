@@ -97,6 +97,18 @@ __device__ inline float block_max(float v, float* scratch) {
     return total;
 }
 
+// The gated activation of a feed-forward, act(gate, up).  limit <= 0: silu(gate) * up.
+// limit > 0: the clamped variant, g = min(gate, limit), u = clamp(up, -limit, limit),
+// g * sigmoid(alpha * g) * (u + 1).
+__device__ inline float glu_act(float g, float u, float limit, float alpha) {
+    if (limit > 0.f) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+    }
+    return g / (1.f + expf(-g)) * u;
+}
+
 static inline int rl_launch_status() {
     return hipGetLastError() == hipSuccess ? RL_OK : RL_ERR_LAUNCH;
 }

@@ -274,15 +274,6 @@ extern "C" int rl_add_rmsnorm_parts(float* residual, const float* parts, int npa
 // limit > 0: the clamped variant, g' = min(g, limit), u' = clamp(u, -limit, limit),
 // g' * sigmoid(alpha * g') * (u' + 1).
 // --------------------------------------------------------------------------- //
-__device__ inline float glu_act(float g, float u, float limit, float alpha) {
-    if (limit > 0.f) {
-        g = fminf(g, limit);
-        u = fminf(fmaxf(u, -limit), limit);
-        return g / (1.f + expf(-alpha * g)) * (u + 1.f);
-    }
-    return g / (1.f + expf(-g)) * u;
-}
-
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter,
                               size_t total, float limit, float alpha) {

@@ -97,6 +97,8 @@ struct SkinnyExtra {
     const float* norm_w;  // [N]
     bf16_t* xt;           // [M, N] residual * norm_w
     float* partial;       // [workgroups][16]
+    // the gated activation of the gate/up variants (limit 0: silu(gate) * up)
+    float glu_limit, glu_alpha;
 };
 
 // LASTQ: groups of four rows of the last tile that belong to the workgroup: 4, or 2 for
@@ -325,7 +327,7 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
                     // path does where the product's result is stored before the activation
                     gate = bf16_to_float(float_to_bf16(gate * scale));
                     up = bf16_to_float(float_to_bf16(up * scale));
-                    v = gate / (1.f + expf(-gate)) * up;
+                    v = glu_act(gate, up, ex.glu_limit, ex.glu_alpha);
                 } else {
                     v = 0.f;
 #pragma unroll
@@ -525,7 +527,7 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_swiglu_stream_kernel(
             // operands rounded to bfloat16, as where the product's result is stored first
             gate = bf16_to_float(float_to_bf16(gate * scale));
             up = bf16_to_float(float_to_bf16(up * scale));
-            out[(size_t)m * ldo + nbase + i] = float_to_bf16(gate / (1.f + expf(-gate)) * up);
+            out[(size_t)m * ldo + nbase + i] = float_to_bf16(glu_act(gate, up, ex.glu_limit, ex.glu_alpha));
         }
     }
 }
@@ -616,11 +618,14 @@ extern "C" int rl_gemm_skinny(const void* X, const void* W, void* out, int M, in
 // -nt tiles: for comparing the two).
 extern "C" int rl_gemm_skinny_swiglu(const void* X, const void* W, void* out, int M, int I, int K,
                                      int ldx, int ldw, int ldo, int nt, int units, const float* x_partial,
-                                     int x_parts, int x_size, float x_eps, hipStream_t stream) {
+                                     int x_parts, int x_size, float x_eps, float glu_limit, float glu_alpha,
+                                     hipStream_t stream) {
     if (M <= 0 || I <= 0) return RL_OK;
     if (!skinny_args_ok(M, K, ldx, ldw) || ldo < I || (x_partial && (x_parts < 1 || x_size < 1)))
         return RL_ERR_ARG;
-    const SkinnyExtra ex = scaled_input(x_partial, x_parts, x_size, x_eps);
+    SkinnyExtra ex = scaled_input(x_partial, x_parts, x_size, x_eps);
+    ex.glu_limit = glu_limit;
+    ex.glu_alpha = glu_alpha;
     int rc = RL_OK;
     if (nt >= 0 && swiglu_stream((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, I, K, ldx, ldw, ldo, units,
                                  ex, stream, &rc))
@@ -811,7 +816,7 @@ extern "C" int rl_gemm_mid_parts(const void* X, const void* W, float* part, int 
 template <int MB, bool SWIGLU>
 __global__ __launch_bounds__(MW* RL_WAVE) void gemm_tile_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, bf16_t* __restrict__ out, int M,
-    int N, int K, int ldx, int ldw, int ldo) {
+    int N, int K, int ldx, int ldw, int ldo, float glu_limit, float glu_alpha) {
     __shared__ __attribute__((aligned(16))) unsigned char xs[2][MB * 16 * WT_PITCH];
     __shared__ __attribute__((aligned(16))) unsigned char wtile[MW][16 * WT_PITCH];
     const int tid = threadIdx.x, lane = tid & (RL_WAVE - 1), wave = tid / RL_WAVE;
@@ -912,7 +917,7 @@ __global__ __launch_bounds__(MW* RL_WAVE) void gemm_tile_kernel(
             for (int i = 0; i < 4; ++i) {
                 const float gate = bf16_to_float(float_to_bf16(acc[mb][i]));
                 const float u = bf16_to_float(float_to_bf16(up[((wave * MB + mb) * 4 + i) * RL_WAVE + lane]));
-                acc[mb][i] = gate / (1.f + expf(-gate)) * u;
+                acc[mb][i] = glu_act(gate, u, glu_limit, glu_alpha);
             }
     }
 #pragma unroll
@@ -938,7 +943,7 @@ __global__ __launch_bounds__(MW* RL_WAVE) void gemm_tile_kernel(
 // out[M, N] = X W^T as bfloat16 (swiglu == 0), or out[M, N] = silu(X Wg^T) * (X Wu^T) with
 // W = [Wg | Wu] stacked by rows, [2N, K].  K a multiple of 128, ldo a multiple of 4.
 extern "C" int rl_gemm_tile(const void* X, const void* W, void* out, int M, int N, int K, int ldx,
-                            int ldw, int ldo, int swiglu, hipStream_t stream) {
+                            int ldw, int ldo, int swiglu, float glu_limit, float glu_alpha, hipStream_t stream) {
     if (M <= 0 || N <= 0) return RL_OK;
     if (K < KSTEP || K % KSTEP || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo % 4 || ldo < N || !out)
         return RL_ERR_ARG;
@@ -954,10 +959,10 @@ extern "C" int rl_gemm_tile(const void* X, const void* W, void* out, int M, int 
     do {                                                                                          \
         if (swiglu)                                                                               \
             hipLaunchKernelGGL((gemm_tile_kernel<MBV, true>), grid, block, 0, stream, x, w, o, M, \
-                               N, K, ldx, ldw, ldo);                                              \
+                               N, K, ldx, ldw, ldo, glu_limit, glu_alpha);                        \
         else                                                                                      \
             hipLaunchKernelGGL((gemm_tile_kernel<MBV, false>), grid, block, 0, stream, x, w, o,   \
-                               M, N, K, ldx, ldw, ldo);                                           \
+                               M, N, K, ldx, ldw, ldo, 0.f, 0.f);                                 \
     } while (0)
     if (mb == 1)
         RL_TILE(1);

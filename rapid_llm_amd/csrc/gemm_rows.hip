@@ -64,7 +64,7 @@ __device__ inline void rows_store4<bf16_t>(bf16_t* p, const float (&v)[4]) {
 template <int TB, int MB, bool SWIGLU, typename OutT, int DEPTH, int NW>
 __global__ __launch_bounds__(NW* RL_WAVE) void gemm_rows_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, OutT* __restrict__ out, int M,
-    int N, int K, int ldx, int ldw, int ldo) {
+    int N, int K, int ldx, int ldw, int ldo, float glu_limit, float glu_alpha) {
     static_assert(TB % DEPTH == 0, "the ring of tiles in flight closes within a chunk");
     static_assert(!SWIGLU || TB % 2 == 0, "gate and up tiles come in pairs");
     constexpr int TPU = SWIGLU ? 2 : 1;  // tiles per unit
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(NW* RL_WAVE) void gemm_rows_kernel(
                     // (rapid_llm/kernels/ops/activation/swiglu.py:91-121)
                     gate = bf16_to_float(float_to_bf16(gate));
                     up = bf16_to_float(float_to_bf16(up));
-                    v[i] = gate / (1.f + expf(-gate)) * up;
+                    v[i] = glu_act(gate, up, glu_limit, glu_alpha);
                 } else {
                     float s = 0.f;
 #pragma unroll
@@ -214,11 +214,16 @@ __global__ __launch_bounds__(NW* RL_WAVE) void gemm_rows_kernel(
     }
 }
 
+// the gated activation of the call being dispatched (limit 0: silu(gate) * up), set by the
+// entry point and handed to the kernel by rows_launch: the host side is one thread a device
+static float rows_glu_limit = 0.f, rows_glu_alpha = 0.f;
+
 template <int TB, int MB, bool SWIGLU, typename OutT, int DEPTH, int NW>
 static int rows_launch(const void* X, const void* W, void* out, int M, int N, int K, int ldx, int ldw,
                        int ldo, int groups, hipStream_t stream) {
     hipLaunchKernelGGL((gemm_rows_kernel<TB, MB, SWIGLU, OutT, DEPTH, NW>), dim3(groups), dim3(NW * RL_WAVE), 0,
-                       stream, (const bf16_t*)X, (const bf16_t*)W, (OutT*)out, M, N, K, ldx, ldw, ldo);
+                       stream, (const bf16_t*)X, (const bf16_t*)W, (OutT*)out, M, N, K, ldx, ldw, ldo,
+                       rows_glu_limit, rows_glu_alpha);
     return rl_launch_status();
 }
 
@@ -256,8 +261,11 @@ extern "C" int rl_gemm_rows_holds(int swiglu, int per_group, int M) {
 // of 16, K a multiple of 128.  `groups` workgroups share the N / 16 units evenly, each at most
 // `per_group` of them (one of rl_gemm_rows_holds).
 extern "C" int rl_gemm_rows(const void* X, const void* W, void* out, int M, int N, int K, int ldx, int ldw,
-                            int ldo, int swiglu, int out_type, int per_group, int groups, hipStream_t stream) {
+                            int ldo, int swiglu, int out_type, int per_group, int groups, float glu_limit,
+                            float glu_alpha, hipStream_t stream) {
     if (M <= 0 || N <= 0) return RL_OK;
+    rows_glu_limit = glu_limit;
+    rows_glu_alpha = glu_alpha;
     if (M > 64 || N % 16 || K < RK || K % RK || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo % 4 || ldo < N ||
         !X || !W || !out || groups < 1)
         return RL_ERR_ARG;

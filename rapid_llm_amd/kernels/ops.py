@@ -300,7 +300,8 @@ def qknorm_rope_kvwrite(
         value_head0 = nq + nkv
     _need(qkv, "qkv", None, (tokens, None))
     row_width = qkv.shape[1]
-    if value_head0 < 0 or row_width < (max(value_head0, nq) + nkv) * d or row_width % 8:
+    if value_head0 < 0 or row_width < (max(value_head0, nq) + nkv) * d or (d % 8 == 0 and row_width % 8):
+        # (heads in steps of 8 channels are read 8 or 16 bytes at a time, so rows must start aligned)
         raise KernelError(
             f"packed rows of {row_width} columns do not hold {nq} query, {nkv} key and {nkv} value heads "
             f"of {d} (values from head {value_head0}) in whole groups of 8 columns"
@@ -628,14 +629,19 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, scaled=N
         raise KernelError(f"scaled rows need the few-row product: {m} rows over {k}")
     if _tile_applies(m, n, k, n):
         out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-        _ok(core().rl_gemm_tile(_p(x), _p(w), _p(out), m, n, k, k, k, n, 0, _stream()), "rl_gemm_tile")
+        _ok(
+            core().rl_gemm_tile(_p(x), _p(w), _p(out), m, n, k, k, k, n, 0, ctypes.c_float(0.0), ctypes.c_float(0.0),
+                                _stream()),
+            "rl_gemm_tile",
+        )
         return out
     plan = rows_plan(m, n, k, swiglu=False)
     if plan is not None:
         wide = torch.float32 if out_dtype == torch.float32 else torch.bfloat16
         out = torch.empty((m, n), dtype=wide, device=x.device)
         _ok(
-            core().rl_gemm_rows(_p(x), _p(w), _p(out), m, n, k, k, k, n, 0, _tag(wide), *plan, _stream()),
+            core().rl_gemm_rows(_p(x), _p(w), _p(out), m, n, k, k, k, n, 0, _tag(wide), *plan, ctypes.c_float(0.0),
+                                ctypes.c_float(0.0), _stream()),
             "rl_gemm_rows",
         )
         return out
@@ -814,11 +820,14 @@ def add_rmsnorm_parts(
     )
 
 
-def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, scaled=None) -> torch.Tensor | None:
-    """``silu(x Wg^T) * (x Wu^T)`` for the packed ``[gate | up]`` matrix in one kernel: for
-    few rows, and for up to 512 rows over a small matrix; ``None`` when the shape is not one a
-    fused kernel takes.  ``scaled``: as in ``gemm_bf16``."""
+def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, scaled=None, limit: float = 0.0,
+                     alpha: float = GLU_ALPHA) -> torch.Tensor | None:
+    """``act(x Wg^T, x Wu^T)`` for the packed ``[gate | up]`` matrix in one kernel: for few rows,
+    and for up to 512 rows over a small matrix; ``None`` when the shape is not one a fused kernel
+    takes.  ``act`` is ``silu(g) * u``, or with a ``limit`` the clamped variant of :func:`swiglu`.
+    ``scaled``: as in ``gemm_bf16``."""
     m, k = x.shape
+    glu = (ctypes.c_float(limit), ctypes.c_float(alpha))
     two_i = w_gate_up.shape[0]
     if k % 8 or two_i % 2 or x.dtype != torch.bfloat16 or w_gate_up.dtype != torch.bfloat16:
         return None
@@ -830,14 +839,14 @@ def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, scaled=None) -> t
         _need(w_gate_up, "w_gate_up", torch.bfloat16, (two_i, k))
         if _tile_applies(m, two_i, k, inter):
             out = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
-            _ok(core().rl_gemm_tile(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, 1, _stream()), "rl_gemm_tile")
+            _ok(core().rl_gemm_tile(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, 1, *glu, _stream()), "rl_gemm_tile")
             return out
         plan = rows_plan(m, inter, k, swiglu=True)
         if plan is None:
             return None
         out = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
         _ok(
-            core().rl_gemm_rows(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, 1, BF16, *plan, _stream()),
+            core().rl_gemm_rows(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, 1, BF16, *plan, *glu, _stream()),
             "rl_gemm_rows",
         )
         return out
@@ -849,7 +858,7 @@ def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, scaled=None) -> t
     _ok(
         core().rl_gemm_skinny_swiglu(
             _p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, nt, chip().units,
-            *_scaled_args(scaled, m, k), _stream()
+            *_scaled_args(scaled, m, k), *glu, _stream()
         ),
         "rl_gemm_skinny_swiglu",
     )

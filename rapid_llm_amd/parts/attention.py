@@ -62,8 +62,10 @@ class GQAAttention(Mixer):
     ) -> None:
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not divisible by {num_kv_heads} kv heads")
-        if head_dim % 8 or not 8 <= head_dim <= 256:
-            raise ValueError(f"attention kernels take head sizes in steps of 8 up to 256, got {head_dim}")
+        if head_dim % 2 or not 2 <= head_dim <= 256:
+            # multiples of 16 run on the matrix cores, every other even size on the kernel that
+            # takes any size (an architecture's configuration may be stricter)
+            raise ValueError(f"attention kernels take even head sizes up to 256, got {head_dim}")
         self.hidden_size = hidden_size
         self.nq, self.nkv, self.d = num_heads, num_kv_heads, head_dim
         self.prefix = checkpoint_prefix
@@ -92,7 +94,7 @@ class GQAAttention(Mixer):
         self.value_head0 = num_heads if self.values_are_keys else num_heads + num_kv_heads
         self.qkv_rows = (num_heads + (1 if self.values_are_keys else 2) * num_kv_heads) * head_dim
         self.gate_rows = num_heads if head_gate_name else 0
-        self.gate_pad = -self.gate_rows % 8
+        self.gate_pad = -(self.qkv_rows + self.gate_rows) % 8 if self.gate_rows else 0
         self.plain_row = not self.values_are_keys and not self.gate_rows
         self.qkv = Linear(hidden_size, self.qkv_rows + self.gate_rows + self.gate_pad)
         self.o = Linear(num_heads * head_dim, hidden_size)

@@ -61,9 +61,11 @@ class SwiGLU(FeedForward):
 
     def forward(self, x, ctx):
         w = self.gate_up.weight
-        if w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and not self.limit:
+        if w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
             # few rows: product and activation in one kernel
-            act = ops.gemm_bf16_swiglu(x.rows, w, scaled=x) if isinstance(x, ScaledRows) else ops.gemm_bf16_swiglu(x, w)
+            glu = dict(limit=self.limit, alpha=self.alpha)
+            act = (ops.gemm_bf16_swiglu(x.rows, w, scaled=x, **glu) if isinstance(x, ScaledRows)
+                   else ops.gemm_bf16_swiglu(x, w, **glu))
             if act is not None:
                 return self.down.deferred(act, ctx)
         gu = self.gate_up(x)

@@ -43,13 +43,13 @@ FOKU_P = {
 }
 PAGE_P = 8
 
-# Q: one head everywhere, a head size between the matrix cores' steps (24), a window of five
+# Q: one head everywhere, a head size that is no multiple of 8 (20), a window of five
 # keys (one page and a bit), a loop of one pass over the first layer only, the smallest sizes
 FOKU_Q = {
     "architecture": "Fokulorn", "width": 64, "vocab": 130, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6},
     "layers": [
         {"type": "mlstm", "mixer": _mem(1, 8, 8, 20.0), "mlp": _mlp(48, 0.75)},
-        {"type": "attention", "mixer": _attn(2, 1, 24, 0.25, 5, (12, 77.0)), "mlp": None},
+        {"type": "attention", "mixer": _attn(2, 1, 20, 0.25, 5, (10, 77.0)), "mlp": None},
     ],
     "loop": {"start": 0, "stop": 1, "times": 1},
 }

@@ -199,6 +199,31 @@ def test_clamped_gated_activation(dtype):
     torch.testing.assert_close(out.float().cpu(), want, **tol)
 
 
+@pytest.mark.parametrize("rows", [1, 8, 16, 17, 40, 64, 200])
+@pytest.mark.parametrize("inter,k", [(256, 128), (1024, 256), (3072, 1024)])
+def test_clamped_activation_inside_the_gate_up_product(rows, inter, k):
+    """Every product kernel that applies the gated activation in its epilogue (few rows, 17 to
+    64 rows, the tile product) against the product followed by the activation on the CPU."""
+    from rapid_llm_amd.kernels import ops
+
+    torch.manual_seed(rows + inter)
+    x = torch.randn(rows, k).bfloat16()
+    w = (torch.randn(2 * inter, k) * (3.0 / k ** 0.5)).bfloat16()
+    for limit in (1.5, 0.0):
+        got = ops.gemm_bf16_swiglu(x.to(DEV), w.to(DEV), limit=limit)
+        if got is None:
+            assert rows > 16  # beyond the few-row kernel not every shape has a fused product
+            return
+        gu = (x.float() @ w.float().T).bfloat16().float()
+        g, u = gu[:, :inter], gu[:, inter:]
+        if limit:
+            g, u = g.clamp(max=limit), u.clamp(-limit, limit)
+            want = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+        else:
+            want = torch.nn.functional.silu(g) * u
+        torch.testing.assert_close(got.float().cpu(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_head_gate_and_scaled_embedding(dtype):
     from rapid_llm_amd.kernels import ops
@@ -219,7 +244,7 @@ def test_head_gate_and_scaled_embedding(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("nq,nkv,d,rot", [(4, 2, 32, 32), (6, 6, 16, 8), (2, 1, 24, 12), (8, 2, 64, 0)])
+@pytest.mark.parametrize("nq,nkv,d,rot", [(4, 2, 32, 32), (6, 6, 16, 8), (2, 1, 24, 12), (3, 1, 20, 10), (8, 2, 64, 0)])
 def test_values_are_the_unrotated_keys_in_the_cache(dtype, nq, nkv, d, rot):
     """The cache write of a packed ``[q | k | gates]`` row: rotated keys (interleaved pairs, the
     first ``rot`` channels) in the key pages, the same keys unrotated in the value pages."""
@@ -227,6 +252,7 @@ def test_values_are_the_unrotated_keys_in_the_cache(dtype, nq, nkv, d, rot):
 
     page, tokens = 8, 21
     width = (nq + nkv) * d + 8
+    width += -width % 8
     packed = torch.randn(tokens, width).to(dtype)
     positions = torch.arange(5, 5 + tokens, dtype=torch.int32)
     table = torch.tensor([[0, 3, 1, 4, 2, 0]], dtype=torch.int32)

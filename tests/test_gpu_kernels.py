@@ -758,7 +758,8 @@ def test_gate_up_product_that_streams_several_pairs_a_workgroup(shape, scaled):
         rc = core.rl_gemm_skinny_swiglu(
             ctypes.c_void_p(xd.data_ptr()), ctypes.c_void_p(wd.data_ptr()), ctypes.c_void_p(out.data_ptr()),
             m, inter, k, k, k, inter, nt, ops.chip().units, ctypes.c_void_p(partial.data_ptr() if scaled else 0),
-            7 if scaled else 0, k if scaled else 0, ctypes.c_float(1e-6), ops._stream())
+            7 if scaled else 0, k if scaled else 0, ctypes.c_float(1e-6), ctypes.c_float(0.0), ctypes.c_float(0.0),
+            ops._stream())
         assert rc == 0
         return out
     streamed, single = run(2), run(-2)
@@ -921,7 +922,7 @@ def test_rows_product_refuses_what_it_was_not_built_for():
     w = torch.zeros((2 * 25600, 256), dtype=torch.bfloat16, device=DEV)
     out = torch.zeros((64, 25600), dtype=torch.bfloat16, device=DEV)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
-    call = lambda m, n, k, sw, per, groups: core.rl_gemm_rows(P(x), P(w), P(out), m, n, k, k, k, n, sw, 1, per, groups, ops._stream())
+    call = lambda m, n, k, sw, per, groups: core.rl_gemm_rows(P(x), P(w), P(out), m, n, k, k, k, n, sw, 1, per, groups, ctypes.c_float(0.0), ctypes.c_float(0.0), ops._stream())
     assert call(64, 25600, 256, 1, 5, 320) == 1   # five pairs beside 64 rows: not built
     assert call(48, 25600, 256, 1, 5, 320) == 0
     assert call(48, 25600, 256, 1, 5, 256) == 1   # a share of seven pairs in a workgroup that holds five
