@@ -609,6 +609,68 @@ __global__ __launch_bounds__(256) void mlstm_chunk_output_kernel(
     }
 }
 
+// The gates' projection: out[t][n] = sum_k x[t][k] w[n][k] in float32, for the few rows of w
+// that a recurrence's gates have (two a head).  One workgroup per token: its 256 threads walk K
+// four channels a thread at a time; sixteen outputs are accumulated side by side and folded over
+// the workgroup at the end.  The weights (a few hundred KB) stay in the caches for every token.
+template <typename T>
+__global__ __launch_bounds__(256) void gate_product_kernel(const T* __restrict__ x, const float* __restrict__ w,
+                                                           float* __restrict__ out, int tokens, int K, int N) {
+    __shared__ float part[4][16];
+    const int lane = threadIdx.x & (RL_WAVE - 1), wave = threadIdx.x / RL_WAVE;
+    const int t = blockIdx.x;
+    const T* row = x + (size_t)t * K;
+    for (int n0 = 0; n0 < N; n0 += 16) {
+        float acc[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+        if (K % 4 == 0) {  // whole groups of four channels: sixteen 16-byte loads at once
+            for (int k = 4 * threadIdx.x; k < K; k += 4 * 256) {
+                float xv[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xv[j] = to_float(row[k + j]);
+                float4 wv[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    wv[i] = *reinterpret_cast<const float4*>(w + (size_t)min(n0 + i, N - 1) * K + k);
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    acc[i] += xv[0] * wv[i].x + xv[1] * wv[i].y + xv[2] * wv[i].z + xv[3] * wv[i].w;
+            }
+        } else {
+            for (int k = threadIdx.x; k < K; k += 256) {
+                const float xv = to_float(row[k]);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[i] += xv * w[(size_t)min(n0 + i, N - 1) * K + k];
+            }
+        }
+        __syncthreads();  // the last round's sums are read
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float total = wave_sum(acc[i]);
+            if (lane == 0) part[wave][i] = total;
+        }
+        __syncthreads();
+        if (threadIdx.x < 16 && n0 + (int)threadIdx.x < N)
+            out[(size_t)t * N + n0 + threadIdx.x] =
+                part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x] + part[3][threadIdx.x];
+    }
+}
+
+extern "C" int rl_gate_product(const void* x, const float* w, float* out, int tokens, int K, int N, int act_type,
+                               hipStream_t stream) {
+    if (tokens <= 0 || N <= 0) return RL_OK;
+    if (K < 1) return RL_ERR_ARG;
+    dim3 grid(tokens), block(256);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(gate_product_kernel<float>, grid, block, 0, stream, (const float*)x, w, out, tokens, K, N);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(gate_product_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)x, w, out, tokens, K, N);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
 extern "C" int rl_mlstm_max_key_dim() { return 256; }
 
 // slices of a column's state rows over lanes: the fewest that leave a lane ML_DREG rows

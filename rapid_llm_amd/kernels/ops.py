@@ -1348,6 +1348,18 @@ def _mlstm_chunks(ctx):
     return found
 
 
+def gate_product(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x w^T`` in float32 for a float32 matrix ``w`` of few rows (the gates of a recurrence,
+    two a head) and rows ``x`` of either type: one launch, no widened copy of ``x``."""
+    tokens, k = x.shape
+    n = w.shape[0]
+    _need(x, "x")
+    _need(w, "gate weights", torch.float32, (n, k))
+    out = torch.empty((tokens, n), dtype=torch.float32, device=x.device)
+    _ok(mlstm_lib().rl_gate_product(_p(x), _p(w), _p(out), tokens, k, n, _tag(x.dtype), _stream()), "rl_gate_product")
+    return out
+
+
 def mlstm(
     packed: torch.Tensor,
     columns: tuple[int, int, int, int],

@@ -14,7 +14,10 @@ by a weight and by ``sigmoid(gate(x))``, and the output projection follows.
 
 One product makes the packed row ``[q | k | v | gate]`` in the compute type.  The gates'
 pre-activations come from a second, small product whose matrix is held in float32 in every
-engine, and everything from there to the finished head outputs is float32 in the kernels
+engine and whose result is float32 (a kernel of its own for these few columns; in a bfloat16
+engine's steps of few rows the few-row product with float32 results, over the same weights as
+bfloat16 where that loses nothing: a product of two bfloat16 numbers is exact in float32), and
+everything from there to the finished head outputs is float32 in the kernels
 (``csrc/mlstm.hip``).  The state lives in the request's slot (``cache.states``), so portions,
 single tokens and batches of both continue where the request's last step stopped.
 """
@@ -90,7 +93,15 @@ class MatrixMemory(Mixer):
 
     def bind(self, params, runtime) -> None:
         self.packed.bind(params[self.name + ".packed"])
-        self.gates.bind(params[self.name + ".gates"])
+        gates = params[self.name + ".gates"]
+        self.gates.bind(gates)
+        # the same weights as bfloat16 for the few-row product, where they are exactly that
+        self.gates_few = None
+        if runtime.dtype == torch.bfloat16 and self.hidden_size % 8 == 0:
+            narrow = gates.to(torch.bfloat16)
+            if torch.equal(narrow.to(torch.float32), gates):
+                self.gates_few = Linear(self.hidden_size, 2 * self.heads)
+                self.gates_few.bind(narrow)
         self.gate_bias = params[self.name + ".gate_bias"]
         self.norm_weight = params[self.name + ".norm"]
         self.o.bind(params[self.name + ".o"])
@@ -107,11 +118,15 @@ class MatrixMemory(Mixer):
 
     @property
     def accepts_scaled_rows(self) -> bool:
-        return False  # two products read the normalised rows
+        # both products that read the normalised rows must be able to finish the norm
+        return self.gates_few is not None and self.packed.takes_scaled_rows()
 
     def forward(self, x, ctx, cache):
         packed = self.packed(x)
-        pre = self.gates(x, out_dtype=torch.float32)
+        if self.gates_few is not None and self.gates_few.skinny(x):
+            pre = self.gates_few(x, out_dtype=torch.float32)
+        else:
+            pre = ops.gate_product(x, self.gates.weight)
         out = torch.empty((x.shape[0], self.heads * self.dv), dtype=packed.dtype, device=x.device)
         ops.mlstm(
             packed, self.columns, pre, self.gate_bias, self.norm_weight, out, ctx,

@@ -111,7 +111,9 @@ def random_params(
         if spec.role == "vector":
             out[spec.name] = _draw(spec.shape, spec.init, gen, std, norm_std, device)
         elif spec.role == "matrix_f32":
-            out[spec.name] = torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
+            # values as a bfloat16 checkpoint would store them, held in float32
+            drawn = torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
+            out[spec.name] = drawn.to(torch.bfloat16).to(torch.float32)
         elif spec.role == "table":
             out[spec.name] = torch.zeros(spec.shape, dtype=torch.int32, device=device)
         else:

@@ -225,6 +225,18 @@ def test_clamped_activation_inside_the_gate_up_product(rows, inter, k):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tokens,k,n", [(1, 96, 6), (37, 70, 2), (300, 1024, 16), (5, 256, 40)])
+def test_gate_projection_in_float32(dtype, tokens, k, n):
+    from rapid_llm_amd.kernels import ops
+
+    x = torch.randn(tokens, k).to(dtype)
+    w = torch.randn(n, k)
+    got = ops.gate_product(x.to(DEV), w.to(DEV))
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got.cpu(), (x.double() @ w.double().T).float(), rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_head_gate_and_scaled_embedding(dtype):
     from rapid_llm_amd.kernels import ops
 
