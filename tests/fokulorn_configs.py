@@ -67,7 +67,23 @@ FOKU_R = {
 }
 PAGE_R = 16
 
-FOKU = {"P": (FOKU_P, PAGE_P, 301), "Q": (FOKU_Q, PAGE_Q, 302), "R": (FOKU_R, PAGE_R, 303)}
+# S: sizes that no vector access divides (width 100 = 4 * 25, feed-forward 50 and 27, vocabulary 97,
+# key sizes 12 and 6, value sizes 10 and 22, an attention head of 18 channels of which 6 rotate): every
+# kernel takes its element-by-element path and the bfloat16 products go to the library; two windows
+# (two pools of pages), one of them a single key; a loop over the last two layers
+FOKU_S = {
+    "architecture": "Fokulorn", "width": 100, "vocab": 97, "embedding": {"scale": 10.0}, "norm": {"eps": 1e-5},
+    "layers": [
+        {"type": "attention", "mixer": _attn(5, 5, 18, 0.3, 1, (6, 3000.0)), "mlp": _mlp(50, 2.0)},
+        {"type": "mlstm", "mixer": _mem(5, 12, 10, 6.0), "mlp": _mlp(27, 1.0)},
+        {"type": "attention", "mixer": _attn(3, 1, 18, 0.2, 33, (18, 100.0)), "mlp": None},
+        {"type": "mlstm", "mixer": _mem(2, 6, 22, 30.0), "mlp": None},
+    ],
+    "loop": {"start": 2, "stop": 4, "times": 2},
+}
+PAGE_S = 8
+
+FOKU = {"P": (FOKU_P, PAGE_P, 301), "Q": (FOKU_Q, PAGE_Q, 302), "R": (FOKU_R, PAGE_R, 303), "S": (FOKU_S, PAGE_S, 304)}
 
 
 def tensor_shapes(cfg) -> dict[str, tuple[int, ...]]:
