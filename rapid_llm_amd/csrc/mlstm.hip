@@ -49,7 +49,7 @@ __global__ __launch_bounds__(1024) void mlstm_gates_kernel(
     const int waves = blockDim.x / RL_WAVE;
     const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
     const int slot = seq_slots[s];
-    float m = m_state[(size_t)slot * heads + h];  // the maximum that enters this round
+    float m = m_state[(size_t)slot * heads + h];  // the maximum that enters these tokens
     const float bi = gate_bias ? gate_bias[h] : 0.f;
     const float bf = gate_bias ? gate_bias[heads + h] : 0.f;
     for (int base = t0; base < t1; base += blockDim.x) {
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(1024) void mlstm_gates_kernel(
                 F = Fu + F;
             }
         }
-        __syncthreads();  // the last round's totals are read
+        __syncthreads();  // the totals of the tokens before are still read
         if (lane == RL_WAVE - 1) {
             wF[wave] = F;
             wG[wave] = G;
@@ -644,7 +644,7 @@ __global__ __launch_bounds__(256) void gate_product_kernel(const T* __restrict__
                 for (int i = 0; i < 16; ++i) acc[i] += xv * w[(size_t)min(n0 + i, N - 1) * K + k];
             }
         }
-        __syncthreads();  // the last round's sums are read
+        __syncthreads();  // the sums of the columns before are still read
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const float total = wave_sum(acc[i]);
