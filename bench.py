@@ -396,6 +396,20 @@ def _time_kernels(z: dict, prompt_len: int, batch: int) -> dict:
         for _ in range(3):
             call()
         torch.cuda.synchronize()
+        if max(lens) == 1:
+            # single tokens: replayed from a graph, as a decode step runs them (launched one
+            # by one the three kernels cost the host more than the device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(10):
+                    call()
+            graph.replay()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for _ in range(5):
+                graph.replay()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t) / 50
         t = time.perf_counter()
         for _ in range(10):
             call()

@@ -26,8 +26,17 @@
 // zero at the start of a request.
 #include "common.h"
 
-#define ML_TOKENS 16   // tokens staged per round of the scan
+// A (token, head) row of the unfinished outputs: dv numerators, then n . q, padded so that
+// every row starts at a multiple of 16 bytes.
+__host__ __device__ inline int raw_width(int dv) { return (dv + 4) & ~3; }
+
+#define ML_TOKENS 16   // tokens staged at a time by the scan
 #define ML_DREG 32     // state rows a lane holds of its column
+
+template <typename T>
+struct alignas(sizeof(T) * 4) Vec4 {
+    T v[4];
+};
 
 __device__ inline float soft_cap(float x, float cap) { return cap * tanhf(x / cap); }
 
@@ -95,7 +104,7 @@ __global__ __launch_bounds__(1024) void mlstm_gates_kernel(
 // One wave per (request, head, block of columns).  A wave's 64 lanes are `slices` groups of
 // `cols` = 64 / slices lanes: lane l holds, of column blockIdx.z * cols + l % cols, the state
 // rows d = l / cols + r * slices (r < ML_DREG).  Column dv is the normaliser n.
-// raw [tokens, heads, dv + 1]: S_t^T q_t (q scaled), the last entry n_t . q_t.
+// raw [tokens, heads, raw_width(dv)]: S_t^T q_t (q scaled), entry dv of a row is n_t . q_t.
 template <typename T>
 __global__ __launch_bounds__(RL_WAVE) void mlstm_scan_kernel(
     const T* __restrict__ packed, int row_width, int q_col, int k_col, int v_col,
@@ -159,7 +168,7 @@ __global__ __launch_bounds__(RL_WAVE) void mlstm_scan_kernel(
                 }
             }
             for (int off = cols; off < RL_WAVE; off <<= 1) acc += __shfl_xor(acc, off, RL_WAVE);
-            if (slice == 0 && live) raw[((size_t)(base + u) * heads + h) * (dv + 1) + j] = acc * q_scale;
+            if (slice == 0 && live) raw[((size_t)(base + u) * heads + h) * raw_width(dv) + j] = acc * q_scale;
         }
     }
     if (live) {
@@ -224,7 +233,7 @@ __global__ __launch_bounds__(256) void mlstm_step_kernel(
     part[wave][lane] = acc;
     __syncthreads();
     if (wave == 0 && live)
-        raw[((size_t)t * heads + h) * (dv + 1) + j] =
+        raw[((size_t)t * heads + h) * raw_width(dv) + j] =
             (part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane]) * q_scale;
 }
 
@@ -239,8 +248,34 @@ __global__ __launch_bounds__(256) void mlstm_finish_kernel(
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int h = blockIdx.y * (blockDim.x / RL_WAVE) + threadIdx.x / RL_WAVE;
     if (h >= heads) return;
-    const float* r = raw + ((size_t)t * heads + h) * (dv + 1);
+    const float* r = raw + ((size_t)t * heads + h) * raw_width(dv);
     const float den = fmaxf(fabsf(r[dv]), expf(-m_tok[(size_t)t * heads + h])) + 1e-6f;
+    const T* gate = packed + (size_t)t * row_width + g_col + (size_t)h * dv;
+    const float* w = weight + (size_t)h * dv;
+    T* dst = out + ((size_t)t * heads + h) * dv;
+    // four channels a lane where every row involved starts on a multiple of four elements
+    if (dv % 4 == 0 && row_width % 4 == 0 && g_col % 4 == 0) {
+        float ss = 0.f;
+        for (int j = 4 * lane; j < dv; j += 4 * RL_WAVE) {
+            const float4 o = *reinterpret_cast<const float4*>(r + j);
+            const float a = o.x / den, b = o.y / den, c = o.z / den, d = o.w / den;
+            ss += a * a + b * b + c * c + d * d;
+        }
+        ss = wave_sum(ss);
+        const float inv = 1.f / sqrtf(ss / (float)dv + eps);
+        for (int j = 4 * lane; j < dv; j += 4 * RL_WAVE) {
+            const float4 o = *reinterpret_cast<const float4*>(r + j);
+            const float4 wv = *reinterpret_cast<const float4*>(w + j);
+            const Vec4<T> gv = *reinterpret_cast<const Vec4<T>*>(gate + j);
+            const float ov[4] = {o.x, o.y, o.z, o.w}, ww[4] = {wv.x, wv.y, wv.z, wv.w};
+            Vec4<T> y;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                y.v[k] = from_float<T>(ov[k] / den * inv * ww[k] / (1.f + expf(-to_float(gv.v[k]))));
+            *reinterpret_cast<Vec4<T>*>(dst + j) = y;
+        }
+        return;
+    }
     float ss = 0.f;
     for (int j = lane; j < dv; j += RL_WAVE) {
         const float o = r[j] / den;
@@ -248,11 +283,9 @@ __global__ __launch_bounds__(256) void mlstm_finish_kernel(
     }
     ss = wave_sum(ss);
     const float inv = 1.f / sqrtf(ss / (float)dv + eps);
-    const T* gate = packed + (size_t)t * row_width + g_col + (size_t)h * dv;
-    T* dst = out + ((size_t)t * heads + h) * dv;
     for (int j = lane; j < dv; j += RL_WAVE) {
         const float g = to_float(gate[j]);
-        dst[j] = from_float<T>(r[j] / den * inv * weight[(size_t)h * dv + j] / (1.f + expf(-g)));
+        dst[j] = from_float<T>(r[j] / den * inv * w[j] / (1.f + expf(-g)));
     }
 }
 
@@ -601,11 +634,11 @@ __global__ __launch_bounds__(256) void mlstm_chunk_output_kernel(
             for (int r = 0; r < 4; ++r) {
                 const int t = 16 * rt + 4 * g + r, j = jw + 16 * ct;
                 if (t < count && j < dv)
-                    raw[((size_t)(begin + t) * heads + h) * (dv + 1) + j] = acc[rt][ct][r] * q_scale;
+                    raw[((size_t)(begin + t) * heads + h) * raw_width(dv) + j] = acc[rt][ct][r] * q_scale;
             }
     if (first && (int)threadIdx.x < count) {
         const int t = threadIdx.x;
-        raw[((size_t)(begin + t) * heads + h) * (dv + 1) + dv] = (sRow[t] + sE[t] * sDot[t]) * q_scale;
+        raw[((size_t)(begin + t) * heads + h) * raw_width(dv) + dv] = (sRow[t] + sE[t] * sDot[t]) * q_scale;
     }
 }
 

@@ -1422,7 +1422,8 @@ def mlstm(
     log_keep = torch.empty((tokens, heads), dtype=torch.float32, device=dev)
     log_take = torch.empty_like(log_keep)
     m_tok = torch.empty_like(log_keep)
-    raw = torch.empty((tokens, heads, dv + 1), dtype=torch.float32, device=dev)
+    # rows of the unfinished outputs: dv numerators, then n . q, padded to a multiple of 16 bytes
+    raw = torch.empty((tokens, heads, (dv + 4) & ~3), dtype=torch.float32, device=dev)
     _ok(
         lib.rl_mlstm_gates(
             _p(gate_pre), _p(gate_bias), _p(ctx.cu_seqlens), _p(ctx.seq_slots), _p(m), _p(log_keep),
