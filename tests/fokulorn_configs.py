@@ -83,7 +83,19 @@ FOKU_S = {
 }
 PAGE_S = 8
 
-FOKU = {"P": (FOKU_P, PAGE_P, 301), "Q": (FOKU_Q, PAGE_Q, 302), "R": (FOKU_R, PAGE_R, 303), "S": (FOKU_S, PAGE_S, 304)}
+# T: recurrent layers only (no pages, no block tables: the cache is state slots alone), looped twice
+FOKU_T = {
+    "architecture": "Fokulorn", "width": 72, "vocab": 150, "embedding": {"scale": 4.0}, "norm": {"eps": 1e-6},
+    "layers": [
+        {"type": "mlstm", "mixer": _mem(3, 24, 16, 9.0), "mlp": _mlp(40, 5.0)},
+        {"type": "mlstm", "mixer": _mem(2, 16, 56, 14.0), "mlp": None},
+    ],
+    "loop": {"start": 0, "stop": 2, "times": 2},
+}
+PAGE_T = 16
+
+FOKU = {"P": (FOKU_P, PAGE_P, 301), "Q": (FOKU_Q, PAGE_Q, 302), "R": (FOKU_R, PAGE_R, 303), "S": (FOKU_S, PAGE_S, 304),
+        "T": (FOKU_T, PAGE_T, 305)}
 
 
 def tensor_shapes(cfg) -> dict[str, tuple[int, ...]]:

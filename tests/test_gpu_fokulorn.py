@@ -302,6 +302,7 @@ LENGTHS = {
     "Q": [1, 4, 5, 6, 9, 33, 80],              # around the window of 5 and the page of 4
     "R": [2, 15, 64, 129, 131, 260],           # around the window of 130
     "S": [1, 2, 17, 33, 34, 35, 90],           # a window of one key; around the window of 33
+    "T": [1, 2, 15, 16, 63, 64, 65, 200],      # around the chunk of 64 and the length from which steps run in chunks
 }
 
 
@@ -353,7 +354,7 @@ def _check(got, want, dtype, label, rounding=None):
         )
 
 
-@pytest.mark.parametrize("which", ["P", "Q", "R", "S"])
+@pytest.mark.parametrize("which", ["P", "Q", "R", "S", "T"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_every_cut_matches_plain(tmp_path, which, dtype):
     cfg, page, seed = FOKU[which]
