@@ -504,7 +504,7 @@ __global__ void qknorm_rope_kvwrite_kernel(
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int d, int rotary_half, int interleaved, float eps,
-    int write_cache, int write_values, int head0, int row_width, int v_head0) {
+    int write_cache, int write_values, int head0, int row_width, int v_head0, const float* bias) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -531,7 +531,9 @@ __global__ void qknorm_rope_kvwrite_kernel(
             const int h = head - nq - nkv;
             const T* xv = row + (size_t)(v_head0 + h) * d;  // where the row keeps this value head
             T* dst = v_cache + ((page * nkv + h) * d) * page_size + off;
-            for (int i = lane; i < d; i += RL_WAVE) dst[(size_t)i * page_size] = xv[i];
+            for (int i = lane; i < d; i += RL_WAVE)
+                dst[(size_t)i * page_size] =
+                    bias ? from_float<T>(to_float(xv[i]) + bias[(size_t)(v_head0 + h) * d + i]) : xv[i];
             continue;
         }
         const bool is_q = head < nq;
@@ -554,6 +556,10 @@ __global__ void qknorm_rope_kvwrite_kernel(
             if (p < half) {
                 x1[r] = to_float(x[e1[r]]);
                 x2[r] = to_float(x[e2[r]]);
+                if (bias) {  // the projection's bias, added here instead of by a kernel of its own
+                    x1[r] += bias[(size_t)head * d + e1[r]];
+                    x2[r] += bias[(size_t)head * d + e2[r]];
+                }
                 ss += x1[r] * x1[r] + x2[r] * x2[r];
             }
         }
@@ -602,7 +608,7 @@ __device__ inline void qknorm_rope_kvwrite_vec(
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values, int head0,
-    int row_width, int v_head0) {
+    int row_width, int v_head0, const float* bias) {
     constexpr int HPW = RL_WAVE / LPH;  // heads per wave
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -627,7 +633,9 @@ __device__ inline void qknorm_rope_kvwrite_vec(
         const int h = head - nq - nkv;
         const T* xv = row + (size_t)(v_head0 + h) * d;
         T* dst = v_cache + ((page * nkv + h) * d) * page_size + off;
-        for (int i = li; i < d; i += LPH) dst[(size_t)i * page_size] = xv[i];
+        for (int i = li; i < d; i += LPH)
+            dst[(size_t)i * page_size] =
+                bias ? from_float<T>(to_float(xv[i]) + bias[(size_t)(v_head0 + h) * d + i]) : xv[i];
         return;
     }
     const bool is_q = head < nq;
@@ -642,6 +650,10 @@ __device__ inline void qknorm_rope_kvwrite_vec(
         for (int k = 0; k < 4; ++k) {
             a[k] = to_float(va.v[k]);
             b[k] = to_float(vb.v[k]);
+            if (bias) {
+                a[k] += bias[(size_t)head * d + 4 * li + k];
+                b[k] += bias[(size_t)head * d + half + 4 * li + k];
+            }
             ss += a[k] * a[k] + b[k] * b[k];
         }
     }
@@ -689,11 +701,11 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_vec_kernel(
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values, int head0,
-    int row_width, int v_head0) {
+    int row_width, int v_head0, const float* bias) {
     qknorm_rope_kvwrite_vec<T, LPH>(blockIdx.x, blockIdx.y, qkv, q_out, k_cache, v_cache, q_norm_w, k_norm_w,
                                     cos_tab, sin_tab, positions, token_slot, block_table, table_stride,
                                     page_size, nq, nkv, d, eps, write_cache, write_values, head0, row_width,
-                                    v_head0);
+                                    v_head0, bias);
 }
 
 template <typename T>
@@ -702,7 +714,7 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
                           const int* positions, const int* token_slot, const int* block_table,
                           int table_stride, int page_size, int tokens, int nq, int nkv, int d,
                           int rotary_half, int interleaved, float eps, int write_cache,
-                          int write_values, int head0, int row_width, int v_head0, hipStream_t stream) {
+                          int write_values, int head0, int row_width, int v_head0, const float* bias, hipStream_t stream) {
     const int total_heads = nq + (write_values ? 2 * nkv : nkv) - head0;  // heads to work on
     // the vectorised kernel: head sizes in steps of 8, the half-split rotation of the whole head
     if (d % 8 == 0 && (!cos_tab || (rotary_half == d / 2 && !interleaved))) {
@@ -714,12 +726,12 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
             hipLaunchKernelGGL((qknorm_rope_kvwrite_vec_kernel<T, 16>), grid, block, 0, stream, qkv,
                                q_out, k_cache, v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab,
                                positions, token_slot, block_table, table_stride, page_size, nq, nkv,
-                               d, eps, write_cache, write_values, head0, row_width, v_head0);
+                               d, eps, write_cache, write_values, head0, row_width, v_head0, bias);
         else
             hipLaunchKernelGGL((qknorm_rope_kvwrite_vec_kernel<T, 32>), grid, block, 0, stream, qkv,
                                q_out, k_cache, v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab,
                                positions, token_slot, block_table, table_stride, page_size, nq, nkv,
-                               d, eps, write_cache, write_values, head0, row_width, v_head0);
+                               d, eps, write_cache, write_values, head0, row_width, v_head0, bias);
         return;
     }
     const int head_groups = (total_heads + 3) / 4;
@@ -727,7 +739,7 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
     hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<T>, grid, block, 0, stream, qkv, q_out, k_cache,
                        v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                        block_table, table_stride, page_size, nq, nkv, d, rotary_half, interleaved, eps,
-                       write_cache, write_values, head0, row_width, v_head0);
+                       write_cache, write_values, head0, row_width, v_head0, bias);
 }
 
 // Values of 16 consecutive tokens of the batch and one kv head, written by one workgroup.
@@ -743,7 +755,7 @@ template <typename T>
 __device__ inline void v_tile_write(
     int tile, int h, const T* __restrict__ qkv, T* __restrict__ v_cache, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int tokens, int nq, int nkv, int d, int row_width, int v_head0) {
+    int page_size, int tokens, int nq, int nkv, int d, int row_width, int v_head0, const float* bias) {
     __shared__ T vt[VT_TOKENS][256 + 8];
     __shared__ int s_page[VT_TOKENS];
     __shared__ int s_off[VT_TOKENS];
@@ -761,8 +773,10 @@ __device__ inline void v_tile_write(
     }
     for (int idx = threadIdx.x; idx < VT_TOKENS * d; idx += 256) {
         const int i = idx / d, c = idx - i * d;
-        if (t0 + i < tokens)
-            vt[i][c] = qkv[(size_t)(t0 + i) * row_width + (size_t)(v_head0 + h) * d + c];
+        if (t0 + i < tokens) {
+            const T v = qkv[(size_t)(t0 + i) * row_width + (size_t)(v_head0 + h) * d + c];
+            vt[i][c] = bias ? from_float<T>(to_float(v) + bias[(size_t)(v_head0 + h) * d + c]) : v;
+        }
     }
     __syncthreads();
     for (int idx = threadIdx.x; idx < 4 * d; idx += 256) {
@@ -800,17 +814,17 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int tokens, int head_groups, int nq, int nkv, int d, float eps, int head0,
-    int row_width, int v_head0) {
+    int row_width, int v_head0, const float* bias) {
     const int qk_blocks = tokens * head_groups;
     if ((int)blockIdx.x < qk_blocks) {
         qknorm_rope_kvwrite_vec<T, LPH>(blockIdx.x / head_groups, blockIdx.x % head_groups, qkv, q_out, k_cache,
                                         v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                                         block_table, table_stride, page_size, nq, nkv, d, eps, 1, 0, head0,
-                                        row_width, v_head0);
+                                        row_width, v_head0, bias);
     } else {
         const int b = blockIdx.x - qk_blocks;
         v_tile_write<T>(b / nkv, b % nkv, qkv, v_cache, positions, token_slot, block_table, table_stride,
-                        page_size, tokens, nq, nkv, d, row_width, v_head0);
+                        page_size, tokens, nq, nkv, d, row_width, v_head0, bias);
     }
 }
 
@@ -818,9 +832,9 @@ template <typename T>
 __global__ __launch_bounds__(256) void v_tile_write_kernel(
     const T* __restrict__ qkv, T* __restrict__ v_cache, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int tokens, int nq, int nkv, int d, int row_width, int v_head0) {
+    int page_size, int tokens, int nq, int nkv, int d, int row_width, int v_head0, const float* bias) {
     v_tile_write<T>(blockIdx.x, blockIdx.y, qkv, v_cache, positions, token_slot, block_table, table_stride,
-                    page_size, tokens, nq, nkv, d, row_width, v_head0);
+                    page_size, tokens, nq, nkv, d, row_width, v_head0, bias);
 }
 
 // true if it launched: head sizes in steps of 8, and a grid that fits
@@ -829,7 +843,7 @@ static bool launch_qkv_prepare(const T* qkv, T* q_out, T* k_cache, T* v_cache, c
                                const float* k_norm_w, const float* cos_tab, const float* sin_tab,
                                const int* positions, const int* token_slot, const int* block_table,
                                int table_stride, int page_size, int tokens, int nq, int nkv, int d,
-                               float eps, int head0, int row_width, int v_head0, hipStream_t stream) {
+                               float eps, int head0, int row_width, int v_head0, const float* bias, hipStream_t stream) {
     if (d % 8) return false;
     const int lph = d <= 128 ? 16 : 32;
     const int heads_per_block = 4 * (RL_WAVE / lph);
@@ -841,12 +855,12 @@ static bool launch_qkv_prepare(const T* qkv, T* q_out, T* k_cache, T* v_cache, c
         hipLaunchKernelGGL((qkv_prepare_kernel<T, 16>), grid, block, 0, stream, qkv, q_out, k_cache, v_cache,
                            q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
                            table_stride, page_size, tokens, head_groups, nq, nkv, d, eps, head0, row_width,
-                           v_head0);
+                           v_head0, bias);
     else
         hipLaunchKernelGGL((qkv_prepare_kernel<T, 32>), grid, block, 0, stream, qkv, q_out, k_cache, v_cache,
                            q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
                            table_stride, page_size, tokens, head_groups, nq, nkv, d, eps, head0, row_width,
-                           v_head0);
+                           v_head0, bias);
     return true;
 }
 
@@ -856,8 +870,7 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
                                       const int* positions, const int* token_slot,
                                       const int* block_table, int table_stride, int page_size,
                                       int tokens, int nq, int nkv, int d, int rotary_half,
-                                      int interleaved, float eps, int write_cache, int row_width,
-                                      int v_head0, int act_type, hipStream_t stream) {
+                                      int interleaved, float eps, int write_cache, int row_width, int v_head0, const float* bias, int act_type, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (d % 2 || d > 256) return RL_ERR_ARG;
     // the packed row: query heads from column 0, key heads behind them, the value heads from
@@ -879,34 +892,34 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
     if (tile_values && whole_split && act_type == RL_F32 &&
         launch_qkv_prepare<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache, q_norm_w,
                                   k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                                  table_stride, page_size, tokens, nq, nkv, d, eps, head0, row_width, v_head0,
+                                  table_stride, page_size, tokens, nq, nkv, d, eps, head0, row_width, v_head0, bias,
                                   stream))
         return rl_launch_status();
     if (tile_values && whole_split && act_type == RL_BF16 &&
         launch_qkv_prepare<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                                    q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                                   table_stride, page_size, tokens, nq, nkv, d, eps, head0, row_width, v_head0,
+                                   table_stride, page_size, tokens, nq, nkv, d, eps, head0, row_width, v_head0, bias,
                                    stream))
         return rl_launch_status();
     if (act_type == RL_F32) {
         launch_qknorm<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache,
                              q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                              block_table, table_stride, page_size, tokens, nq, nkv, d, rotary_half,
-                             interleaved, eps, write_cache, !tile_values, head0, row_width, v_head0, stream);
+                             interleaved, eps, write_cache, !tile_values, head0, row_width, v_head0, bias, stream);
         if (tile_values)
             hipLaunchKernelGGL(v_tile_write_kernel<float>, vgrid, block, 0, stream,
                                (const float*)qkv, (float*)v_cache, positions, token_slot,
-                               block_table, table_stride, page_size, tokens, nq, nkv, d, row_width, v_head0);
+                               block_table, table_stride, page_size, tokens, nq, nkv, d, row_width, v_head0, bias);
     } else if (act_type == RL_BF16) {
         launch_qknorm<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
                               (bf16_t*)v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions,
                               token_slot, block_table, table_stride, page_size, tokens, nq, nkv, d,
                               rotary_half, interleaved, eps, write_cache, !tile_values, head0, row_width,
-                              v_head0, stream);
+                              v_head0, bias, stream);
         if (tile_values)
             hipLaunchKernelGGL(v_tile_write_kernel<bf16_t>, vgrid, block, 0, stream,
                                (const bf16_t*)qkv, (bf16_t*)v_cache, positions, token_slot,
-                               block_table, table_stride, page_size, tokens, nq, nkv, d, row_width, v_head0);
+                               block_table, table_stride, page_size, tokens, nq, nkv, d, row_width, v_head0, bias);
     } else {
         return RL_ERR_ARG;
     }

@@ -13,15 +13,22 @@
 // here is float32: gates, maxima, decays, state and outputs; the element type only decides how
 // the packed projections are read and the finished rows are stored.
 //
-// Three kernels a step:
-//   gates   one wave per (request, head): i, f, the maxima m_t, and per token the logarithms
-//           of the two decay factors (log keep = f_t + m_{t-1} - m_t, log take = i_t - m_t,
-//           both <= 0 up to rounding).  Activations side by side, the max-plus recurrence
-//           as a scan over the workgroup.
-//   scan    per (request, head, block of columns): the state update and S^T q token by token,
-//           the tokens' rows staged through LDS sixteen at a time.
+// A step runs the gates kernel, one of three forms of the recurrence, and the finishing kernel:
+//   gates   one workgroup per (request, head): i, f, the maxima m_t, and per token the
+//           logarithms of the two decay factors (log keep = f_t + m_{t-1} - m_t, log take =
+//           i_t - m_t, both <= 0 up to rounding).  Activations side by side, the max-plus
+//           recurrence as a scan over the workgroup.
+//   step    every request brings one token: per (token, head, 64 columns) the state is read,
+//           updated and written back once, as a stream.
+//   scan    short portions: per (request, head, block of columns) the state stays in registers
+//           and the tokens' rows are staged through LDS sixteen at a time.
+//   chunked portions of prompts: chunks of 64 tokens on the float32 matrix instruction, three
+//           kernels (every chunk's own sum, the carry over a request's chunks, every chunk's
+//           outputs); described where they stand.
 //   finish  per (token, head): the division, the head's unit root mean square, the weight over
 //           all heads' channels and the sigmoid gate.
+// The gates' pre-activations come from gate_product (or from the few-row product of the core
+// library) as float32.
 // State per request slot: S [slot, head, dk, dv], n [slot, head, dk], m [slot, head], float32,
 // zero at the start of a request.
 #include "common.h"
@@ -704,6 +711,8 @@ extern "C" int rl_gate_product(const void* x, const float* w, float* out, int to
     return rl_launch_status();
 }
 
+// the largest key size the kernels take (the step and scan kernels stage a head's query and
+// key in LDS, the chunk kernels hold up to sixteen tiles of state rows a wave)
 extern "C" int rl_mlstm_max_key_dim() { return 256; }
 
 // slices of a column's state rows over lanes: the fewest that leave a lane ML_DREG rows

@@ -86,6 +86,11 @@ def mlstm_lib() -> ctypes.CDLL:
     global _mlstm
     if _mlstm is None:
         _mlstm = build.load(build.mlstm_library())
+        if _mlstm.rl_mlstm_max_key_dim() != MLSTM_MAX_KEY_DIM:
+            raise KernelError(
+                f"the recurrence library takes key sizes up to {_mlstm.rl_mlstm_max_key_dim()}, "
+                f"the launch rules expect {MLSTM_MAX_KEY_DIM}"
+            )
     return _mlstm
 
 
@@ -280,6 +285,7 @@ def qknorm_rope_kvwrite(
     max_position: int,
     pairing: str = "half_split",
     value_head0: Optional[int] = None,
+    bias: Optional[torch.Tensor] = None,
 ) -> None:
     """Norm + rotate q and k, write k and v to the cache pages (skipped when the caches
     are ``None``: a layer that reads another layer's cache).  ``q_out`` ``None``: the query
@@ -292,7 +298,9 @@ def qknorm_rope_kvwrite(
     A packed row holds the query heads, then the key heads, and the value heads from head
     ``value_head0`` on (default ``nq + nkv``, right behind the keys; ``nq``: the values are the
     keys as projected, before the rotation); it may be wider than that (columns of the same
-    product that another kernel reads)."""
+    product that another kernel reads).  ``bias`` (float32, one entry a column of the packed
+    row): the projection's bias, added to the heads as they are read, before norm and rotation,
+    instead of by a kernel of its own after the product."""
     if pairing not in ROTARY_PAIRINGS:
         raise KernelError(f"rotation pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
     tokens = qkv.shape[0]
@@ -335,12 +343,14 @@ def qknorm_rope_kvwrite(
             raise KernelError(
                 f"position {max_position} is beyond the rotation table of {cos.shape[0]} positions"
             )
+    if bias is not None:
+        _need(bias, "bias of the packed projection", torch.float32, (row_width,))
     _ok(
         core().rl_qknorm_rope_kvwrite(
             _p(qkv), _p(q_out), _p(k_cache), _p(v_cache), _p(q_norm_w), _p(k_norm_w), _p(cos),
             _p(sin), _p(positions), _p(token_slot), _p(block_table), block_table.stride(0),
             page_size, tokens, nq, nkv, d, half, ROTARY_PAIRINGS[pairing], ctypes.c_float(eps), int(write),
-            row_width, value_head0, _tag(qkv.dtype), _stream(),
+            row_width, value_head0, _p(bias), _tag(qkv.dtype), _stream(),
         ),
         "rl_qknorm_rope_kvwrite",
     )

@@ -145,7 +145,13 @@ class GQAAttention(Mixer):
         return specs
 
     def bind(self, params, runtime) -> None:
-        self.qkv.bind(params[self.name + ".qkv"], params[self.name + ".qkv_bias"] if self.qkv_bias else None)
+        bias = params[self.name + ".qkv_bias"] if self.qkv_bias else None
+        # A plain [q | k | v] row may run through kernels that read the packed row themselves
+        # (the fused decode step, queries finished inside the attention kernels): its bias is
+        # added after the product.  Any other row always passes the kernel that norms, rotates
+        # and writes the cache, which adds the bias as it reads the heads.
+        self.bias_in_kernel = None if self.plain_row else bias
+        self.qkv.bind(params[self.name + ".qkv"], bias if self.plain_row else None)
         self.o.bind(params[self.name + ".o"], params[self.name + ".o_bias"] if self.o_bias else None)
         if self.qk_norm_eps is not None:
             self.q_norm_w = params[self.name + ".q_norm"]
@@ -194,7 +200,7 @@ class GQAAttention(Mixer):
             cache.v if cache.owns_pages else None,
             self.q_norm_w, self.k_norm_w, cos, sin,
             ctx.positions, ctx.token_slot, table, cache.page_size,
-            self.nq, self.nkv, self.d, eps, ctx.max_position, pairing, self.value_head0,
+            self.nq, self.nkv, self.d, eps, ctx.max_position, pairing, self.value_head0, self.bias_in_kernel,
         )
         ops.paged_attention(
             qkv if in_kernel else q, cache.k, cache.v, out, ctx, table, cache.page_size,

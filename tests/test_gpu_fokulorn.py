@@ -257,9 +257,11 @@ def test_head_gate_and_scaled_embedding(dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nq,nkv,d,rot", [(4, 2, 32, 32), (6, 6, 16, 8), (2, 1, 24, 12), (3, 1, 20, 10), (8, 2, 64, 0)])
-def test_values_are_the_unrotated_keys_in_the_cache(dtype, nq, nkv, d, rot):
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_values_are_the_unrotated_keys_in_the_cache(dtype, nq, nkv, d, rot, with_bias):
     """The cache write of a packed ``[q | k | gates]`` row: rotated keys (interleaved pairs, the
-    first ``rot`` channels) in the key pages, the same keys unrotated in the value pages."""
+    first ``rot`` channels) in the key pages, the same keys unrotated in the value pages; the
+    projection's bias, when the kernel is given it, is added before either."""
     from rapid_llm_amd.kernels import ops
 
     page, tokens = 8, 21
@@ -275,12 +277,13 @@ def test_values_are_the_unrotated_keys_in_the_cache(dtype, nq, nkv, d, rot):
     if rot:
         inv = 1.0 / (500.0 ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))
         cos, sin = ops.rope_table(inv.to(DEV), 64)
+    bias = torch.randn(width) if with_bias else None
     ops.qknorm_rope_kvwrite(
         packed.to(DEV), q_out, k_cache, v_cache, None, None, cos, sin, positions.to(DEV),
         torch.zeros(tokens, dtype=torch.int32, device=DEV), table.to(DEV), page, nq, nkv, d, 0.0,
-        int(positions.max()), "interleaved", value_head0=nq,
+        int(positions.max()), "interleaved", value_head0=nq, bias=bias.to(DEV) if with_bias else None,
     )
-    x = packed.float()
+    x = packed.float() + (bias if with_bias else 0.0)
     q = x[:, : nq * d].view(tokens, nq, d)
     k = x[:, nq * d:(nq + nkv) * d].view(tokens, nkv, d)
     q_want, k_want = (plain_rotate_interleaved(a, positions, rot, 500.0) if rot else a for a in (q, k))
@@ -291,6 +294,19 @@ def test_values_are_the_unrotated_keys_in_the_cache(dtype, nq, nkv, d, rot):
         pg, slot = int(table[0, pos // page]), pos % page
         torch.testing.assert_close(k_cache[pg, :, slot].float().cpu(), k_want[t], **tol)
         torch.testing.assert_close(v_cache[pg, :, :, slot].float().cpu(), k[t].to(dtype).float(), rtol=0, atol=0)
+    # fewer than eight tokens take the kernel that writes the values head by head
+    few = 3
+    v_few = torch.zeros_like(v_cache)
+    ops.qknorm_rope_kvwrite(
+        packed[:few].contiguous().to(DEV), q_out[:few].contiguous(), torch.zeros_like(k_cache), v_few, None, None, cos,
+        sin, positions[:few].contiguous().to(DEV), torch.zeros(few, dtype=torch.int32, device=DEV), table.to(DEV), page,
+        nq, nkv, d, 0.0, int(positions[:few].max()), "interleaved", value_head0=nq,
+        bias=bias.to(DEV) if with_bias else None,
+    )
+    for t in range(few):
+        pos = int(positions[t])
+        torch.testing.assert_close(v_few[int(table[0, pos // page]), :, :, pos % page].float().cpu(),
+                                   k[t].to(dtype).float(), rtol=0, atol=0)
 
 
 # --------------------------------------------------------------------------- #
