@@ -1,7 +1,8 @@
 """Host side of the cache: pages, block tables and per-request state slots.  Device-free.
 
 Keys and values live in pages of ``page_size`` positions.  Layers with the same needs form
-a *group* (all keys, or a window of them); each group has a page pool and one block table
+a *group* (all keys, or a window of them, with or without a number of first positions that
+stay readable behind the window); each group has a page pool and one block table
 row per request slot: ``table[slot, i]`` is the page holding positions
 ``[i * page_size, (i + 1) * page_size)`` of the request in that slot, or the null page 0.
 Pages come back when a request ends and, in a windowed group, as soon as the window has
@@ -74,11 +75,13 @@ class PagePool:
 
 @dataclass(frozen=True)
 class GroupSpec:
-    """Layers that share page ids.  ``window`` 0: every position is kept."""
+    """Layers that share page ids.  ``window`` 0: every position is kept.  With a window,
+    the pages of the first ``keep_first`` positions are never given back before the request ends."""
 
     group_id: int
     window: int
     layers: tuple[int, ...]
+    keep_first: int = 0
 
 
 @dataclass
@@ -147,11 +150,25 @@ class CacheManager:
         if not self._free_slots:
             return None
         slot = self._free_slots.pop()
-        self._requests[request_id] = _Request(request_id, slot, trimmed=[0] * len(self.groups))
+        # a group's kept first pages lie below what trimming may ever touch
+        self._requests[request_id] = _Request(request_id, slot, trimmed=[self._kept_pages(g) for g in self.groups])
         self.fresh_slots.add(slot)
         return slot
 
     # ------------------------------------------------------------------ pages
+    def _kept_pages(self, group: GroupSpec) -> int:
+        """Pages at the head of a request that a windowed group never gives back."""
+        if group.window <= 0 or group.keep_first <= 0:
+            return 0
+        return -(-group.keep_first // self.page_size)
+
+    def _needed_pages(self, group: GroupSpec, trimmed: int, start: int, last: int) -> list[int]:
+        """Indices below ``last`` of the pages that a span beginning at position ``start`` writes
+        or reads: the kept first pages, and everything from the window of ``start`` on."""
+        first = max(trimmed, self._first_needed_page(group, start))
+        kept = min(self._kept_pages(group), first, last)
+        return list(range(kept)) + list(range(first, last))
+
     def _first_needed_page(self, group: GroupSpec, next_position: int) -> int:
         """Index of the first page a query at ``next_position`` or later can still read."""
         if group.window <= 0:
@@ -167,9 +184,8 @@ class CacheManager:
         need = {}
         last = -(-upto // self.page_size)  # pages [0, last) must be addressable
         for gi, g in enumerate(self.groups):
-            first = max(req.trimmed[gi], self._first_needed_page(g, start))
             row = self.tables[g.group_id][req.slot]
-            need[g.group_id] = int(np.count_nonzero(row[first:last] == NULL_PAGE)) if last > first else 0
+            need[g.group_id] = sum(1 for i in self._needed_pages(g, req.trimmed[gi], start, last) if row[i] == NULL_PAGE)
         return need
 
     def reserve(self, request_id: str, upto: int, start: int | None = None) -> bool:
@@ -198,9 +214,8 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             if need[g.group_id] == 0:
                 continue
-            first = max(req.trimmed[gi], self._first_needed_page(g, start))
             row = self.tables[g.group_id][req.slot]
-            holes = [i for i in range(first, last) if row[i] == NULL_PAGE]
+            holes = [i for i in self._needed_pages(g, req.trimmed[gi], start, last) if row[i] == NULL_PAGE]
             pages = self.pools[g.group_id].take(len(holes))
             assert pages is not None
             for i, page in zip(holes, pages):

@@ -60,16 +60,16 @@ class LayerCache:
 
 
 def plan_groups(needs: list[CacheNeed]) -> tuple[list[GroupSpec], list[int | None]]:
-    """Group layers by what they keep (all keys / a window of w).  Returns the groups and,
+    """Group layers by what they keep (all keys / a window of w, with k kept first positions).  Returns the groups and,
     per layer, its group id (``None`` for layers without paged cache).  A layer that shares
     another layer's cache joins that layer's group."""
-    keys: dict[int, int] = {}  # window -> group id
+    keys: dict[tuple[int, int], int] = {}  # (window, kept first positions) -> group id
     layers_of: dict[int, list[int]] = {}
     group_of: list[int | None] = [None] * len(needs)
     for i, need in enumerate(needs):
         if need.kind != "paged" or need.share_with is not None:
             continue
-        gid = keys.setdefault(need.window, len(keys))
+        gid = keys.setdefault((need.window, need.keep_first if need.window else 0), len(keys))
         layers_of.setdefault(gid, []).append(i)
         group_of[i] = gid
     for i, need in enumerate(needs):
@@ -82,15 +82,16 @@ def plan_groups(needs: list[CacheNeed]) -> tuple[list[GroupSpec], list[int | Non
                     f"layer {i} shares the cache of layer {src} but names other paged tensors: "
                     f"{need.paged} against {needs[src].paged}"
                 )
-            if needs[src].window != need.window:
+            if (needs[src].window, needs[src].keep_first) != (need.window, need.keep_first):
                 raise ValueError(
-                    f"layer {i} (window {need.window}) shares the cache of layer {src} "
-                    f"(window {needs[src].window}): a shared cache must keep the same positions"
+                    f"layer {i} (window {need.window}, {need.keep_first} kept) shares the cache of layer {src} "
+                    f"(window {needs[src].window}, {needs[src].keep_first} kept): a shared cache must keep the "
+                    "same positions"
                 )
             group_of[i] = group_of[src]
             layers_of[group_of[i]].append(i)
     windows = {gid: w for w, gid in keys.items()}
-    groups = [GroupSpec(gid, windows[gid], tuple(layers_of[gid])) for gid in sorted(windows)]
+    groups = [GroupSpec(gid, windows[gid][0], tuple(layers_of[gid]), windows[gid][1]) for gid in sorted(windows)]
     return groups, group_of
 
 

@@ -37,6 +37,8 @@ _LAZY: dict[str, str] = {
     "qwen3": "rapid_llm_amd.models.qwen3",
     "Fokulorn": "rapid_llm_amd.models.fokulorn",
     "fokulorn": "rapid_llm_amd.models.fokulorn",
+    "Sikevik": "rapid_llm_amd.models.sikevik",
+    "sikevik": "rapid_llm_amd.models.sikevik",
 }
 
 

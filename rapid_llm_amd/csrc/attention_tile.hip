@@ -1,0 +1,342 @@
+// Paged causal attention over tiles of 16 rows for mixers that the other attention kernels do
+// not take: value heads of a size of their own, a sliding window that keeps a request's first
+// positions visible, and a softmax with one more term in its denominator.  Compiled for one
+// pair of head sizes RL_HEAD_DIM (queries and keys) and RL_VALUE_DIM (values), multiples of 16,
+// in float32 (v_mfma_f32_16x16x4_f32: true 32-bit) and in bfloat16 (v_mfma_f32_16x16x16_bf16,
+// float32 accumulation, scores and softmax state in float32, the weights rounded to bfloat16
+// for the product with the values).
+//
+// One workgroup of AW waves per (tile of 16 rows, kv head).  Rows are (token, query head of
+// the kv group) pairs of ONE request, so grouped heads and neighbouring tokens share every key
+// that is read; a single token's tile holds the heads of its group.  The key tiles are dealt to
+// the waves by their absolute index (tile i goes to wave i % AW), each wave keeps a softmax
+// state of its own, and the states are folded in the order of the waves.  The transposed
+// products are computed,
+//   S^T[keys, rows] = K[keys, d] Q^T[d, rows],   O^T[dv, rows] += V^T[dv, keys] P^T[keys, rows],
+// which leaves a lane with the scores of keys 4g .. 4g + 3 of its own row: exactly its operand
+// of the second product, whose other operand is one read of the transposed value cache.
+//
+// What a row sees: key j of its request with j <= p (its position) and, with a window w > 0,
+// p - j < w or j < keep_first.  The tiles walked are those of [0, keep_first) and those from
+// the window of the tile's first row up to its last row's position.  With `sink` the softmax's
+// denominator is 1 + sum_j exp(s_j): a key of score 0 that carries no value.
+//
+// A row's result does not depend on the tile it falls in, on the other rows there, or on how a
+// prompt was cut into steps: keys are taken in tiles of 16 at absolute positions 0, 16, ..,
+// each wave takes its tiles in ascending order; within a tile the order of every sum is fixed
+// by the key's position; a tile that holds no visible key of a row leaves that row's state as
+// it is, exactly (factor 1, terms 0), and so does a wave without visible keys in the fold.
+// Masked keys contribute exactly zero; pages between the kept positions and the window may have
+// been given back, so what is read there is never multiplied into a sum.
+#include "common.h"
+
+#ifndef RL_HEAD_DIM
+#error "compile with -DRL_HEAD_DIM=<size of a query or key head>"
+#endif
+#ifndef RL_VALUE_DIM
+#error "compile with -DRL_VALUE_DIM=<size of a value head>"
+#endif
+
+namespace tileattn {
+
+constexpr int D = RL_HEAD_DIM;
+constexpr int DV = RL_VALUE_DIM;
+constexpr int DB = D / 16;   // 16-channel chunks of the first product
+constexpr int VB = DV / 16;  // 16-channel blocks of the output
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// what a lane holds of an operand: four consecutive elements
+template <typename T>
+struct Quad;
+template <>
+struct Quad<float> {
+    typedef f32x4 type;
+};
+template <>
+struct Quad<bf16_t> {
+    typedef s16x4 type;
+};
+
+template <typename T>
+__device__ inline typename Quad<T>::type ld_quad(const T* p) {
+    return *reinterpret_cast<const typename Quad<T>::type*>(p);
+}
+
+// acc[16 x 16] += A[16 x 4 quads] B[4 quads x 16]: float32 in four instructions of one element
+// a lane each, bfloat16 in one instruction of four
+__device__ inline f32x4 mma(f32x4 a, f32x4 b, f32x4 acc) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], b[j], acc, 0, 0, 0);
+    return acc;
+}
+__device__ inline f32x4 mma(s16x4 a, s16x4 b, f32x4 acc) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, acc, 0, 0, 0);
+}
+
+__device__ inline void to_quad(const f32x4& p, f32x4& out) { out = p; }
+__device__ inline void to_quad(const f32x4& p, s16x4& out) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = (short)float_to_bf16(p[i]).bits;
+}
+__device__ inline float quad_elem(const f32x4& q, int i) { return q[i]; }
+__device__ inline void store_quad(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+__device__ inline void store_quad(bf16_t* p, f32x4 v) {
+    s16x4 o;
+    to_quad(v, o);
+    *reinterpret_cast<s16x4*>(p) = o;
+}
+
+// the four lanes (r, g = 0..3) that share a row: the same bits in each of them
+__device__ inline float row_max(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16, RL_WAVE));
+    return fmaxf(v, __shfl_xor(v, 32, RL_WAVE));
+}
+__device__ inline float row_sum(float v) {
+    v += __shfl_xor(v, 16, RL_WAVE);
+    return v + __shfl_xor(v, 32, RL_WAVE);
+}
+
+// tile_info: [tiles][3] = index of the request's first token in the step, its tokens in the
+// step, first row of the tile.  The request's first position is read from `positions`.
+template <typename T, int AW>
+__global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    T* __restrict__ out, const int* __restrict__ tile_info, const int* __restrict__ positions,
+    const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
+    int page_size, int nq, int nkv, int window, int keep_first, int sink, float scale) {
+    typedef typename Quad<T>::type quad;
+    const int tile = blockIdx.x;
+    const int hk = blockIdx.y;
+    const int G = nq / nkv;
+    const int at = tile_info[3 * tile], n = tile_info[3 * tile + 1], row0 = tile_info[3 * tile + 2];
+    __shared__ float fold_ml[AW - 1][2][RL_WAVE];
+    __shared__ float fold_acc[AW - 1][VB * 4][RL_WAVE];
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    const int wave = threadIdx.x / RL_WAVE;
+    const int r16 = lane & 15;
+    const int g = lane >> 4;
+    const int start = positions[at];
+    const int* table = block_table + (size_t)token_slot[at] * table_stride;
+
+    const int rows = n * G;
+    const int row = row0 + r16;
+    const bool row_ok = row < rows;
+    const int tok = (row_ok ? row : rows - 1) / G;
+    const int head = hk * G + (row_ok ? row : rows - 1) % G;
+    const int pos = start + tok;
+    const int kend = pos + 1;
+    const int kstart = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int keep = window > 0 ? keep_first : 0;  // keys below it are seen from anywhere
+
+    // the keys any row of the tile sees: the kept first ones, and from the first row's first key
+    // (rows ascend with the tokens), in whole tiles of 16, up to the last row's own position
+    const int first_pos = start + row0 / G;
+    const int last_pos = start + (min(rows, row0 + 16) - 1) / G;
+    const int first_key = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+    const int lo = first_key & ~15;
+    const int hi = last_pos + 1;                     // keys below hi are in the cache
+    const int kept_end = min((keep + 15) & ~15, lo);  // tiles [0, kept_end) come before those of [lo, hi)
+
+    // Q^T: lane (row r16, g) holds channels 16c + 4g .. + 3 of its row
+    quad qf[DB];
+    {
+        const T* qrow = q + ((size_t)(at + tok) * nq + head) * D + 4 * g;
+#pragma unroll
+        for (int c = 0; c < DB; ++c) {
+            qf[c] = ld_quad<T>(qrow + 16 * c);
+            if (!row_ok) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) qf[c][i] = 0;
+            }
+        }
+    }
+
+    float m = -INFINITY, l = 0.f;
+    f32x4 acc[VB];
+#pragma unroll
+    for (int b = 0; b < VB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    // operands of one tile of 16 keys: lane (key r16, g) reads channels 16c + 4g .. + 3 of its
+    // key; lane (channel r16, g) reads keys kb + 4g .. + 3 of its channel in every block
+    struct Frags {
+        quad k[DB], v[VB];
+    };
+    auto load = [&](int kb, Frags& f) {
+        const int key = min(kb + r16, hi - 1);  // beyond the cache: any real key, masked below
+        const T* krow =
+            k_cache + (((size_t)table[key / page_size] * nkv + hk) * page_size + key % page_size) * D + 4 * g;
+#pragma unroll
+        for (int c = 0; c < DB; ++c) f.k[c] = ld_quad<T>(krow + 16 * c);
+        const int key4 = min(kb + 4 * g, (hi - 1) & ~3);
+        const T* vrow = v_cache + (((size_t)table[key4 / page_size] * nkv + hk) * DV + r16) * page_size +
+                        key4 % page_size;
+#pragma unroll
+        for (int b = 0; b < VB; ++b) f.v[b] = ld_quad<T>(vrow + (size_t)16 * b * page_size);
+    };
+
+    // S^T = K Q^T of one tile, the chunks dealt to four accumulators that are added at the
+    // end (one chain of dependent instructions would leave the matrix core idle)
+    auto scores = [&](const Frags& f) -> f32x4 {
+        f32x4 part[4];
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) part[a4] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < DB; ++c) part[c & 3] = mma(f.k[c], qf[c], part[c & 3]);
+        return (part[0] + part[1]) + (part[2] + part[3]);
+    };
+
+    // softmax and second product of the tile at kb, given its scores and its values
+    auto finish_tile = [&](int kb, f32x4 s, const quad (&vcur)[VB]) {
+        // ---- this lane's keys kb + 4g + i of its own row ------------------------------------
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int key = kb + 4 * g + i;
+            const bool seen = row_ok && key < kend && (key >= kstart || key < keep);
+            s[i] = seen ? s[i] * scale : -INFINITY;
+            tmax = fmaxf(tmax, s[i]);
+        }
+        tmax = row_max(tmax);
+        const float m_new = fmaxf(m, tmax);
+        float alpha = 1.f;  // no visible key so far and none here: nothing changes
+        f32x4 p = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (m_new != -INFINITY) {
+            alpha = expf(m - m_new);  // m = -inf before the row's first key: 0
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p[i] = expf(s[i] - m_new);  // masked: exactly 0
+        }
+        l = l * alpha + row_sum((p[0] + p[1]) + (p[2] + p[3]));
+        m = m_new;
+        quad pq;
+        to_quad(p, pq);
+        // ---- O^T = O^T alpha + V^T P^T --------------------------------------------------------
+#pragma unroll
+        for (int b = 0; b < VB; ++b) {
+            quad vf = vcur[b];
+            // keys no row of the tile sees (beyond the cache, or between the kept ones and the
+            // window, whose pages may have been given back) may hold anything: 0 * it must be 0
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kb + 4 * g + i;
+                if (key >= hi || (key < first_key && key >= keep)) vf[i] = 0;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[b][i] *= alpha;
+            acc[b] = mma(vf, pq, acc[b]);
+        }
+    };
+
+    // The wave's tiles, in ascending order: those of the kept keys with index % AW == wave,
+    // then those of [lo, hi) with index % AW == wave.
+    constexpr int STEP = 16 * AW;
+    const int kept_mine = 16 * wave;
+    const int kept_tiles = kept_mine < kept_end ? (kept_end - kept_mine + STEP - 1) / STEP : 0;
+    const int mine = lo + 16 * ((wave - lo / 16) & (AW - 1));  // first tile >= lo with index % AW == wave
+    const int late_tiles = mine < hi ? (hi - mine + STEP - 1) / STEP : 0;
+    const int total = kept_tiles + late_tiles;
+    auto kb_of = [&](int i) -> int {
+        return i < kept_tiles ? kept_mine + i * STEP : mine + (i - kept_tiles) * STEP;
+    };
+    // Software pipeline over the wave's tiles: while a tile goes through softmax and the second
+    // product, the scores of the next have been multiplied and the operands of the one after
+    // are in flight.  The last two tiles stand outside the loop, so that inside it the loads
+    // are issued without a condition.
+    if (total > 0) {
+        int left = total;  // tiles of this wave, the current one included
+        int i = 0;
+        Frags nxt;
+        quad vcur[VB], vnext[VB];
+        load(kb_of(0), nxt);
+        f32x4 sc = scores(nxt);
+#pragma unroll
+        for (int b = 0; b < VB; ++b) vcur[b] = nxt.v[b];
+        if (left > 1) load(kb_of(1), nxt);
+        while (left > 2) {
+            const f32x4 s_next = scores(nxt);
+#pragma unroll
+            for (int b = 0; b < VB; ++b) vnext[b] = nxt.v[b];
+            load(kb_of(i + 2), nxt);
+            __builtin_amdgcn_sched_barrier(0);
+            finish_tile(kb_of(i), sc, vcur);
+            sc = s_next;
+#pragma unroll
+            for (int b = 0; b < VB; ++b) vcur[b] = vnext[b];
+            ++i;
+            --left;
+        }
+        if (left == 2) {
+            const f32x4 s_next = scores(nxt);
+            finish_tile(kb_of(i), sc, vcur);
+            finish_tile(kb_of(i + 1), s_next, nxt.v);
+        } else {
+            finish_tile(kb_of(i), sc, vcur);
+        }
+    }
+    // ---- fold the waves' states in their order (a wave without visible keys has m = -inf,
+    // l = 0 and zero sums: it changes nothing, exactly) ----------------------------------------
+    if (wave > 0) {
+        fold_ml[wave - 1][0][lane] = m;
+        fold_ml[wave - 1][1][lane] = l;
+#pragma unroll
+        for (int b = 0; b < VB; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fold_acc[wave - 1][4 * b + i][lane] = acc[b][i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < AW - 1; ++w) {
+        const float m_w = fold_ml[w][0][lane], l_w = fold_ml[w][1][lane];
+        const float m_new = fmaxf(m, m_w);
+        if (m_new == -INFINITY) continue;
+        const float fa = expf(m - m_new), fb = expf(m_w - m_new);
+        l = l * fa + l_w * fb;
+#pragma unroll
+        for (int b = 0; b < VB; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[b][i] = acc[b][i] * fa + fold_acc[w][4 * b + i][lane] * fb;
+        m = m_new;
+    }
+    if (!row_ok) return;
+    // the key of score 0 that has no value: exp(0 - m) more in the denominator
+    if (sink) l += expf(-m);
+    // acc[b][i] is channel 16b + 4g + i of the lane's row
+    T* orow = out + ((size_t)(at + tok) * nq + head) * DV + 4 * g;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int b = 0; b < VB; ++b)
+        store_quad(orow + 16 * b, (f32x4){acc[b][0] * inv, acc[b][1] * inv, acc[b][2] * inv, acc[b][3] * inv});
+}
+
+}  // namespace tileattn
+
+extern "C" int rl_attn_tile_head_dim() { return tileattn::D; }
+extern "C" int rl_attn_tile_value_dim() { return tileattn::DV; }
+
+// Every token of the step, single tokens and portions alike.  page_size must be a multiple
+// of 4 (the four keys of a lane lie in one page).
+extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_cache, void* out,
+                            const int* tile_info, int num_tiles, const int* positions,
+                            const int* token_slot, const int* block_table, int table_stride,
+                            int page_size, int nq, int nkv, int window, int keep_first, int sink,
+                            float scale, int act_type, hipStream_t stream) {
+    if (num_tiles <= 0) return RL_OK;
+    if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535 || window < 0 || keep_first < 0)
+        return RL_ERR_ARG;
+    constexpr int AW = 4;
+    dim3 grid(num_tiles, nkv), block(AW * RL_WAVE);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL((tileattn::attn_tile_kernel<float, AW>), grid, block, 0, stream, (const float*)q,
+                           (const float*)k_cache, (const float*)v_cache, (float*)out, tile_info, positions,
+                           token_slot, block_table, table_stride, page_size, nq, nkv, window, keep_first, sink,
+                           scale);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW>), grid, block, 0, stream, (const bf16_t*)q,
+                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_info, positions,
+                           token_slot, block_table, table_stride, page_size, nq, nkv, window, keep_first, sink,
+                           scale);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}

@@ -6,15 +6,25 @@
 // --------------------------------------------------------------------------- //
 // embedding: residual[t, :] = table[ids[t], :] * scale   (float32 residual stream)
 // rapid_llm/modules/vocab_parallel.py:102-103
+// With `inv_freq` (hidden / 2 float32 frequencies) a sinusoidal position vector is added:
+// channel 2i gets sin(a), channel 2i + 1 cos(a), a = positions[t] * inv_freq[i] as a float32
+// product; sine and cosine of that angle are evaluated in double.
 // --------------------------------------------------------------------------- //
+__device__ inline float sinusoid_channel(int pos, int channel, const float* __restrict__ inv_freq) {
+    const float angle = (float)pos * inv_freq[channel >> 1];
+    return (float)((channel & 1) ? cos((double)angle) : sin((double)angle));
+}
+
 // A negative id -(r + 1) stands for "the token chosen in row r of the previous step", which
 // the host may not have seen yet: it is read from `fed` (the sampling kernels' output)
 // (rapid_llm/engine/scheduler.py:241-249: the placeholder a device-side gather replaces).
 template <typename W>
 __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ fed, int fed_rows,
                              const W* __restrict__ table, float* __restrict__ out, int hidden,
-                             int vocab, float scale) {
+                             int vocab, float scale, const int* __restrict__ positions,
+                             const float* __restrict__ inv_freq) {
     const int t = blockIdx.x;
+    const int pos = inv_freq ? positions[t] : 0;
     int id = ids[t];
     if (id < 0 && fed && -id - 1 < fed_rows) id = fed[-id - 1];
     // ids are validated on the host; an id outside the table reads row 0 rather than faulting
@@ -29,27 +39,39 @@ __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict_
         for (int i = threadIdx.x * VEC; i < hidden; i += blockDim.x * VEC) {
             const Pack p = *reinterpret_cast<const Pack*>(row + i);
 #pragma unroll
-            for (int j = 0; j < VEC; j += 4)
-                *reinterpret_cast<float4*>(dst + i + j) =
-                    make_float4(to_float(p.v[j]) * scale, to_float(p.v[j + 1]) * scale,
-                                to_float(p.v[j + 2]) * scale, to_float(p.v[j + 3]) * scale);
+            for (int j = 0; j < VEC; j += 4) {
+                float4 v = make_float4(to_float(p.v[j]) * scale, to_float(p.v[j + 1]) * scale,
+                                       to_float(p.v[j + 2]) * scale, to_float(p.v[j + 3]) * scale);
+                if (inv_freq) {
+                    v.x += sinusoid_channel(pos, i + j, inv_freq);
+                    v.y += sinusoid_channel(pos, i + j + 1, inv_freq);
+                    v.z += sinusoid_channel(pos, i + j + 2, inv_freq);
+                    v.w += sinusoid_channel(pos, i + j + 3, inv_freq);
+                }
+                *reinterpret_cast<float4*>(dst + i + j) = v;
+            }
         }
         return;
     }
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]) * scale;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = to_float(row[i]) * scale;
+        if (inv_freq) v += sinusoid_channel(pos, i, inv_freq);
+        dst[i] = v;
+    }
 }
 
 extern "C" int rl_embed(const int* ids, const int* fed, int fed_rows, const void* table,
                         int table_type, float* out, int tokens, int hidden, int vocab, float scale,
-                        hipStream_t stream) {
+                        const int* positions, const float* inv_freq, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
+    if (inv_freq && !positions) return RL_ERR_ARG;
     dim3 grid(tokens), block(256);
     if (table_type == RL_F32)
         hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, fed, fed_rows,
-                           (const float*)table, out, hidden, vocab, scale);
+                           (const float*)table, out, hidden, vocab, scale, positions, inv_freq);
     else if (table_type == RL_BF16)
         hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, fed, fed_rows,
-                           (const bf16_t*)table, out, hidden, vocab, scale);
+                           (const bf16_t*)table, out, hidden, vocab, scale, positions, inv_freq);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -183,6 +205,115 @@ extern "C" int rl_add_rmsnorm(float* residual, const void* delta, const float* w
     else if (act_type == RL_BF16)
         launch_add_rmsnorm<bf16_t>(residual, (const bf16_t*)delta, weight, (bf16_t*)out, rows,
                                    out_rows, hidden, eps, stream);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
+// A sub-layer whose output passes a norm of its own before it joins the stream:
+//   residual += y * rsqrt(mean(y^2) + eps_y) * w_y        (float32, in place)
+//   out       = residual * rsqrt(mean(residual^2) + eps) * w   (skipped when out is null)
+// One block per produced row, `rows` as in rl_add_rmsnorm.  Both statistics and the sum are
+// float32; y is read once and stays in registers between its two passes (rows of up to
+// 8 * blockDim elements, else it is read again).
+// --------------------------------------------------------------------------- //
+template <typename T, int PER>
+__global__ void normed_add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ y,
+                                          const float* __restrict__ w_y, float eps_y,
+                                          const float* __restrict__ weight, T* __restrict__ out,
+                                          const int* __restrict__ rows, int hidden, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int row = rows ? rows[r] : r;
+    float* res = residual + (size_t)row * hidden;
+    const T* yr = y + (size_t)row * hidden;
+    float val[PER];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < PER; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        val[c] = i < hidden ? to_float(yr[i]) : 0.f;
+        ss += val[c] * val[c];
+    }
+    for (int i = threadIdx.x + PER * blockDim.x; i < hidden; i += blockDim.x) {
+        const float v = to_float(yr[i]);
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float rr_y = rsqrtf(ss / (float)hidden + eps_y);
+    float s2 = 0.f;
+#pragma unroll
+    for (int c = 0; c < PER; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < hidden) {
+            val[c] = res[i] + val[c] * rr_y * w_y[i];
+            res[i] = val[c];
+            s2 += val[c] * val[c];
+        }
+    }
+    for (int i = threadIdx.x + PER * blockDim.x; i < hidden; i += blockDim.x) {
+        const float v = res[i] + to_float(yr[i]) * rr_y * w_y[i];
+        res[i] = v;
+        s2 += v * v;
+    }
+    if (!out) return;
+    s2 = block_sum(s2, scratch);
+    const float rrms = rsqrtf(s2 / (float)hidden + eps);
+    T* o = out + (size_t)r * hidden;
+#pragma unroll
+    for (int c = 0; c < PER; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < hidden) o[i] = from_float<T>(val[c] * rrms * weight[i]);
+    }
+    // each thread re-reads exactly the elements it wrote above
+    for (int i = threadIdx.x + PER * blockDim.x; i < hidden; i += blockDim.x)
+        o[i] = from_float<T>(res[i] * rrms * weight[i]);
+}
+
+extern "C" int rl_normed_add_rmsnorm(float* residual, const void* y, const float* w_y, float eps_y,
+                                     const float* weight, void* out, const int* rows, int out_rows,
+                                     int hidden, float eps, int act_type, hipStream_t stream) {
+    if (out_rows <= 0) return RL_OK;
+    if (out && !weight) return RL_ERR_ARG;
+    dim3 grid(out_rows);
+    const int threads = hidden >= 4096 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 256 : 64));
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL((normed_add_rmsnorm_kernel<float, 8>), grid, dim3(threads), 0, stream, residual,
+                           (const float*)y, w_y, eps_y, weight, (float*)out, rows, hidden, eps);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL((normed_add_rmsnorm_kernel<bf16_t, 8>), grid, dim3(threads), 0, stream, residual,
+                           (const bf16_t*)y, w_y, eps_y, weight, (bf16_t*)out, rows, hidden, eps);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
+// out[t] = [a[t] | b[t]] in the compute type: two float32 streams of `hidden` channels side by
+// side, the operand of a product over both.
+template <typename T>
+__global__ void pair_rows_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                 T* __restrict__ out, size_t total, int hidden) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; idx < total; idx += step) {
+        const size_t t = idx / (2 * (size_t)hidden);
+        const int c = (int)(idx - t * 2 * (size_t)hidden);
+        out[idx] = from_float<T>(c < hidden ? a[t * hidden + c] : b[t * hidden + c - hidden]);
+    }
+}
+
+extern "C" int rl_pair_rows(const float* a, const float* b, void* out, int tokens, int hidden,
+                            int act_type, hipStream_t stream) {
+    if (tokens <= 0 || hidden <= 0) return RL_OK;
+    const size_t total = (size_t)tokens * 2 * hidden;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    dim3 grid((unsigned)blocks), block(256);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(pair_rows_kernel<float>, grid, block, 0, stream, a, b, (float*)out, total, hidden);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(pair_rows_kernel<bf16_t>, grid, block, 0, stream, a, b, (bf16_t*)out, total, hidden);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -347,6 +478,106 @@ extern "C" int rl_swiglu(const void* gate_up, void* out, int tokens, int inter, 
 }
 
 // --------------------------------------------------------------------------- //
+// One-operand activations of a two-layer feed-forward, out = act(x):
+//   kind 0: gelu in its tanh form, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+//   kind 1: relu(z)^2
+// With `route` (float32 [tokens, experts]) the first experts * ff columns of a row are the
+// hidden units of `experts` experts side by side, and expert e's units are multiplied by
+// route[t, e] (0 for an expert the token does not use); columns beyond (a shared expert's)
+// pass with the activation alone.
+// --------------------------------------------------------------------------- //
+__device__ inline float unary_act(float z, int kind) {
+    if (kind == 1) {
+        const float r = fmaxf(z, 0.f);
+        return r * r;
+    }
+    return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename T>
+__global__ void unary_act_kernel(const T* __restrict__ x, T* __restrict__ out, size_t total, int cols,
+                                 int kind, const float* __restrict__ route, int experts, int ff) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; idx < total; idx += step) {
+        float v = unary_act(to_float(x[idx]), kind);
+        if (route) {
+            const size_t t = idx / cols;
+            const int c = (int)(idx - t * cols);
+            if (c < experts * ff) v *= route[t * experts + c / ff];
+        }
+        out[idx] = from_float<T>(v);
+    }
+}
+
+extern "C" int rl_unary_act(const void* x, void* out, int tokens, int cols, int kind, const float* route,
+                            int experts, int ff, int act_type, hipStream_t stream) {
+    if (tokens <= 0 || cols <= 0) return RL_OK;
+    if (kind < 0 || kind > 1) return RL_ERR_ARG;
+    if (route && (experts < 1 || ff < 1 || (long)experts * ff > cols)) return RL_ERR_ARG;
+    const size_t total = (size_t)tokens * cols;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    dim3 grid((unsigned)blocks), block(256);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(unary_act_kernel<float>, grid, block, 0, stream, (const float*)x, (float*)out, total,
+                           cols, kind, route, experts, ff);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(unary_act_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)x, (bf16_t*)out,
+                           total, cols, kind, route, experts, ff);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
+// Router of a mixture of experts, one thread a token, float32 throughout:
+//   s = softmax(z) over all experts; the `top` largest are chosen (the lower index wins a tie);
+//   route[t, e] = s_e / (sum of the chosen s + 1e-20) * scale for a chosen expert, else 0.
+// z is overwritten by route.
+// --------------------------------------------------------------------------- //
+#define ROUTE_MAX_EXPERTS 1024
+__global__ void route_kernel(float* __restrict__ z, int tokens, int experts, int top, float scale) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= tokens) return;
+    float* row = z + (size_t)t * experts;
+    float m = -INFINITY;
+    for (int e = 0; e < experts; ++e) m = fmaxf(m, row[e]);
+    float total = 0.f;
+    for (int e = 0; e < experts; ++e) {
+        const float p = expf(row[e] - m);
+        row[e] = p;
+        total += p;
+    }
+    unsigned chosen[ROUTE_MAX_EXPERTS / 32];
+    for (int w = 0; w < (experts + 31) / 32; ++w) chosen[w] = 0u;
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+        int best = -1;
+        float best_s = -1.f;
+        for (int e = 0; e < experts; ++e) {
+            if (chosen[e >> 5] >> (e & 31) & 1u) continue;
+            if (row[e] > best_s) {
+                best_s = row[e];
+                best = e;
+            }
+        }
+        chosen[best >> 5] |= 1u << (best & 31);
+        sum += best_s / total;
+    }
+    const float inv = scale / (sum + 1e-20f);
+    for (int e = 0; e < experts; ++e)
+        row[e] = (chosen[e >> 5] >> (e & 31) & 1u) ? row[e] / total * inv : 0.f;
+}
+
+extern "C" int rl_route(float* z, int tokens, int experts, int top, float scale, hipStream_t stream) {
+    if (tokens <= 0) return RL_OK;
+    if (experts < 1 || experts > ROUTE_MAX_EXPERTS || top < 1 || top > experts) return RL_ERR_ARG;
+    hipLaunchKernelGGL(route_kernel, dim3((tokens + 63) / 64), dim3(64), 0, stream, z, tokens, experts, top, scale);
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
 // cast between float32 and bfloat16 (either direction, or a copy)
 // --------------------------------------------------------------------------- //
 template <typename S, typename D>
@@ -492,7 +723,8 @@ extern "C" int rl_rope_table(const float* inv_freq, float* cos_out, float* sin_o
 //
 // Cache layout of one layer, page p, kv head h:
 //   keys   K[p][h][slot_in_page][d]      (row-major, d contiguous)
-//   values V[p][h][d][slot_in_page]      (transposed: the page's positions contiguous)
+//   values V[p][h][dv][slot_in_page]     (transposed: the page's positions contiguous; a value
+//                                         head has dv channels, which need not be d)
 // A token at position pos of a request lies in page table[slot_of_request][pos / P] at
 // slot_in_page = pos % P.
 // --------------------------------------------------------------------------- //
@@ -504,7 +736,7 @@ __global__ void qknorm_rope_kvwrite_kernel(
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int d, int rotary_half, int interleaved, float eps,
-    int write_cache, int write_values, int head0, int row_width, int v_head0, const float* bias) {
+    int write_cache, int write_values, int head0, int row_width, int v_col0, int dv, const float* bias) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -529,11 +761,11 @@ __global__ void qknorm_rope_kvwrite_kernel(
             // value head: copy into the transposed page (unless the tile kernel below does it)
             if (!write_cache || !write_values) continue;
             const int h = head - nq - nkv;
-            const T* xv = row + (size_t)(v_head0 + h) * d;  // where the row keeps this value head
-            T* dst = v_cache + ((page * nkv + h) * d) * page_size + off;
-            for (int i = lane; i < d; i += RL_WAVE)
+            const T* xv = row + v_col0 + (size_t)h * dv;  // where the row keeps this value head
+            T* dst = v_cache + ((page * nkv + h) * dv) * page_size + off;
+            for (int i = lane; i < dv; i += RL_WAVE)
                 dst[(size_t)i * page_size] =
-                    bias ? from_float<T>(to_float(xv[i]) + bias[(size_t)(v_head0 + h) * d + i]) : xv[i];
+                    bias ? from_float<T>(to_float(xv[i]) + bias[v_col0 + (size_t)h * dv + i]) : xv[i];
             continue;
         }
         const bool is_q = head < nq;
@@ -608,7 +840,7 @@ __device__ inline void qknorm_rope_kvwrite_vec(
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values, int head0,
-    int row_width, int v_head0, const float* bias) {
+    int row_width, int v_col0, int dv, const float* bias) {
     constexpr int HPW = RL_WAVE / LPH;  // heads per wave
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -631,11 +863,11 @@ __device__ inline void qknorm_rope_kvwrite_vec(
     if (head >= nq + nkv) {
         if (!write_cache) return;
         const int h = head - nq - nkv;
-        const T* xv = row + (size_t)(v_head0 + h) * d;
-        T* dst = v_cache + ((page * nkv + h) * d) * page_size + off;
-        for (int i = li; i < d; i += LPH)
+        const T* xv = row + v_col0 + (size_t)h * dv;
+        T* dst = v_cache + ((page * nkv + h) * dv) * page_size + off;
+        for (int i = li; i < dv; i += LPH)
             dst[(size_t)i * page_size] =
-                bias ? from_float<T>(to_float(xv[i]) + bias[(size_t)(v_head0 + h) * d + i]) : xv[i];
+                bias ? from_float<T>(to_float(xv[i]) + bias[v_col0 + (size_t)h * dv + i]) : xv[i];
         return;
     }
     const bool is_q = head < nq;
@@ -701,11 +933,11 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_vec_kernel(
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values, int head0,
-    int row_width, int v_head0, const float* bias) {
+    int row_width, int v_col0, int dv, const float* bias) {
     qknorm_rope_kvwrite_vec<T, LPH>(blockIdx.x, blockIdx.y, qkv, q_out, k_cache, v_cache, q_norm_w, k_norm_w,
                                     cos_tab, sin_tab, positions, token_slot, block_table, table_stride,
                                     page_size, nq, nkv, d, eps, write_cache, write_values, head0, row_width,
-                                    v_head0, bias);
+                                    v_col0, dv, bias);
 }
 
 template <typename T>
@@ -714,7 +946,7 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
                           const int* positions, const int* token_slot, const int* block_table,
                           int table_stride, int page_size, int tokens, int nq, int nkv, int d,
                           int rotary_half, int interleaved, float eps, int write_cache,
-                          int write_values, int head0, int row_width, int v_head0, const float* bias, hipStream_t stream) {
+                          int write_values, int head0, int row_width, int v_col0, int dv, const float* bias, hipStream_t stream) {
     const int total_heads = nq + (write_values ? 2 * nkv : nkv) - head0;  // heads to work on
     // the vectorised kernel: head sizes in steps of 8, the half-split rotation of the whole head
     if (d % 8 == 0 && (!cos_tab || (rotary_half == d / 2 && !interleaved))) {
@@ -726,12 +958,12 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
             hipLaunchKernelGGL((qknorm_rope_kvwrite_vec_kernel<T, 16>), grid, block, 0, stream, qkv,
                                q_out, k_cache, v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab,
                                positions, token_slot, block_table, table_stride, page_size, nq, nkv,
-                               d, eps, write_cache, write_values, head0, row_width, v_head0, bias);
+                               d, eps, write_cache, write_values, head0, row_width, v_col0, dv, bias);
         else
             hipLaunchKernelGGL((qknorm_rope_kvwrite_vec_kernel<T, 32>), grid, block, 0, stream, qkv,
                                q_out, k_cache, v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab,
                                positions, token_slot, block_table, table_stride, page_size, nq, nkv,
-                               d, eps, write_cache, write_values, head0, row_width, v_head0, bias);
+                               d, eps, write_cache, write_values, head0, row_width, v_col0, dv, bias);
         return;
     }
     const int head_groups = (total_heads + 3) / 4;
@@ -739,7 +971,7 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
     hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<T>, grid, block, 0, stream, qkv, q_out, k_cache,
                        v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                        block_table, table_stride, page_size, nq, nkv, d, rotary_half, interleaved, eps,
-                       write_cache, write_values, head0, row_width, v_head0, bias);
+                       write_cache, write_values, head0, row_width, v_col0, dv, bias);
 }
 
 // Values of 16 consecutive tokens of the batch and one kv head, written by one workgroup.
@@ -755,7 +987,7 @@ template <typename T>
 __device__ inline void v_tile_write(
     int tile, int h, const T* __restrict__ qkv, T* __restrict__ v_cache, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int tokens, int nq, int nkv, int d, int row_width, int v_head0, const float* bias) {
+    int page_size, int tokens, int nq, int nkv, int d, int row_width, int v_col0, int dv, const float* bias) {
     __shared__ T vt[VT_TOKENS][256 + 8];
     __shared__ int s_page[VT_TOKENS];
     __shared__ int s_off[VT_TOKENS];
@@ -771,15 +1003,15 @@ __device__ inline void v_tile_write(
         s_page[threadIdx.x] = page;
         s_off[threadIdx.x] = off;
     }
-    for (int idx = threadIdx.x; idx < VT_TOKENS * d; idx += 256) {
-        const int i = idx / d, c = idx - i * d;
+    for (int idx = threadIdx.x; idx < VT_TOKENS * dv; idx += 256) {
+        const int i = idx / dv, c = idx - i * dv;
         if (t0 + i < tokens) {
-            const T v = qkv[(size_t)(t0 + i) * row_width + (size_t)(v_head0 + h) * d + c];
-            vt[i][c] = bias ? from_float<T>(to_float(v) + bias[(size_t)(v_head0 + h) * d + c]) : v;
+            const T v = qkv[(size_t)(t0 + i) * row_width + v_col0 + (size_t)h * dv + c];
+            vt[i][c] = bias ? from_float<T>(to_float(v) + bias[v_col0 + (size_t)h * dv + c]) : v;
         }
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < 4 * d; idx += 256) {
+    for (int idx = threadIdx.x; idx < 4 * dv; idx += 256) {
         const int quarter = idx & 3, c = idx >> 2;
         const int i0 = 4 * quarter;
         const int page = s_page[i0], off = s_off[i0];
@@ -791,13 +1023,13 @@ __device__ inline void v_tile_write(
             Vec4<T> v;
 #pragma unroll
             for (int k = 0; k < 4; ++k) v.v[k] = vt[i0 + k][c];
-            *reinterpret_cast<Vec4<T>*>(v_cache + (((size_t)page * nkv + h) * d + c) * page_size + off) = v;
+            *reinterpret_cast<Vec4<T>*>(v_cache + (((size_t)page * nkv + h) * dv + c) * page_size + off) = v;
         } else {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const int pg = s_page[i0 + k];
                 if (pg >= 0)
-                    v_cache[(((size_t)pg * nkv + h) * d + c) * page_size + s_off[i0 + k]] = vt[i0 + k][c];
+                    v_cache[(((size_t)pg * nkv + h) * dv + c) * page_size + s_off[i0 + k]] = vt[i0 + k][c];
             }
         }
     }
@@ -814,17 +1046,17 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int tokens, int head_groups, int nq, int nkv, int d, float eps, int head0,
-    int row_width, int v_head0, const float* bias) {
+    int row_width, int v_col0, int dv, const float* bias) {
     const int qk_blocks = tokens * head_groups;
     if ((int)blockIdx.x < qk_blocks) {
         qknorm_rope_kvwrite_vec<T, LPH>(blockIdx.x / head_groups, blockIdx.x % head_groups, qkv, q_out, k_cache,
                                         v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                                         block_table, table_stride, page_size, nq, nkv, d, eps, 1, 0, head0,
-                                        row_width, v_head0, bias);
+                                        row_width, v_col0, dv, bias);
     } else {
         const int b = blockIdx.x - qk_blocks;
         v_tile_write<T>(b / nkv, b % nkv, qkv, v_cache, positions, token_slot, block_table, table_stride,
-                        page_size, tokens, nq, nkv, d, row_width, v_head0, bias);
+                        page_size, tokens, nq, nkv, d, row_width, v_col0, dv, bias);
     }
 }
 
@@ -832,9 +1064,9 @@ template <typename T>
 __global__ __launch_bounds__(256) void v_tile_write_kernel(
     const T* __restrict__ qkv, T* __restrict__ v_cache, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int tokens, int nq, int nkv, int d, int row_width, int v_head0, const float* bias) {
+    int page_size, int tokens, int nq, int nkv, int d, int row_width, int v_col0, int dv, const float* bias) {
     v_tile_write<T>(blockIdx.x, blockIdx.y, qkv, v_cache, positions, token_slot, block_table, table_stride,
-                    page_size, tokens, nq, nkv, d, row_width, v_head0, bias);
+                    page_size, tokens, nq, nkv, d, row_width, v_col0, dv, bias);
 }
 
 // true if it launched: head sizes in steps of 8, and a grid that fits
@@ -843,7 +1075,7 @@ static bool launch_qkv_prepare(const T* qkv, T* q_out, T* k_cache, T* v_cache, c
                                const float* k_norm_w, const float* cos_tab, const float* sin_tab,
                                const int* positions, const int* token_slot, const int* block_table,
                                int table_stride, int page_size, int tokens, int nq, int nkv, int d,
-                               float eps, int head0, int row_width, int v_head0, const float* bias, hipStream_t stream) {
+                               float eps, int head0, int row_width, int v_col0, int dv, const float* bias, hipStream_t stream) {
     if (d % 8) return false;
     const int lph = d <= 128 ? 16 : 32;
     const int heads_per_block = 4 * (RL_WAVE / lph);
@@ -855,12 +1087,12 @@ static bool launch_qkv_prepare(const T* qkv, T* q_out, T* k_cache, T* v_cache, c
         hipLaunchKernelGGL((qkv_prepare_kernel<T, 16>), grid, block, 0, stream, qkv, q_out, k_cache, v_cache,
                            q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
                            table_stride, page_size, tokens, head_groups, nq, nkv, d, eps, head0, row_width,
-                           v_head0, bias);
+                           v_col0, dv, bias);
     else
         hipLaunchKernelGGL((qkv_prepare_kernel<T, 32>), grid, block, 0, stream, qkv, q_out, k_cache, v_cache,
                            q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
                            table_stride, page_size, tokens, head_groups, nq, nkv, d, eps, head0, row_width,
-                           v_head0, bias);
+                           v_col0, dv, bias);
     return true;
 }
 
@@ -870,12 +1102,14 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
                                       const int* positions, const int* token_slot,
                                       const int* block_table, int table_stride, int page_size,
                                       int tokens, int nq, int nkv, int d, int rotary_half,
-                                      int interleaved, float eps, int write_cache, int row_width, int v_head0, const float* bias, int act_type, hipStream_t stream) {
+                                      int interleaved, float eps, int write_cache, int row_width, int v_col0, int dv, const float* bias, int act_type, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (d % 2 || d > 256) return RL_ERR_ARG;
-    // the packed row: query heads from column 0, key heads behind them, the value heads from
-    // head v_head0 on (nq + nkv: behind the keys; nq: the values are the unrotated keys)
-    if (v_head0 < 0 || row_width < (nq + nkv) * d || (v_head0 + nkv) * d > row_width) return RL_ERR_ARG;
+    // the packed row: query heads from column 0, key heads behind them, the nkv value heads of dv
+    // channels from column v_col0 on ((nq + nkv) * d: behind the keys; nq * d: the values are the
+    // unrotated keys)
+    if (dv < 1 || dv > 256 || v_col0 < 0 || row_width < (nq + nkv) * d || v_col0 + nkv * dv > row_width)
+        return RL_ERR_ARG;
     // q_out null: the attention kernels finish the query heads themselves, and the work here
     // starts at the first key head
     const int head0 = q_out ? 0 : nq;
@@ -892,34 +1126,34 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
     if (tile_values && whole_split && act_type == RL_F32 &&
         launch_qkv_prepare<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache, q_norm_w,
                                   k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                                  table_stride, page_size, tokens, nq, nkv, d, eps, head0, row_width, v_head0, bias,
+                                  table_stride, page_size, tokens, nq, nkv, d, eps, head0, row_width, v_col0, dv, bias,
                                   stream))
         return rl_launch_status();
     if (tile_values && whole_split && act_type == RL_BF16 &&
         launch_qkv_prepare<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                                    q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                                   table_stride, page_size, tokens, nq, nkv, d, eps, head0, row_width, v_head0, bias,
+                                   table_stride, page_size, tokens, nq, nkv, d, eps, head0, row_width, v_col0, dv, bias,
                                    stream))
         return rl_launch_status();
     if (act_type == RL_F32) {
         launch_qknorm<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache,
                              q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                              block_table, table_stride, page_size, tokens, nq, nkv, d, rotary_half,
-                             interleaved, eps, write_cache, !tile_values, head0, row_width, v_head0, bias, stream);
+                             interleaved, eps, write_cache, !tile_values, head0, row_width, v_col0, dv, bias, stream);
         if (tile_values)
             hipLaunchKernelGGL(v_tile_write_kernel<float>, vgrid, block, 0, stream,
                                (const float*)qkv, (float*)v_cache, positions, token_slot,
-                               block_table, table_stride, page_size, tokens, nq, nkv, d, row_width, v_head0, bias);
+                               block_table, table_stride, page_size, tokens, nq, nkv, d, row_width, v_col0, dv, bias);
     } else if (act_type == RL_BF16) {
         launch_qknorm<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
                               (bf16_t*)v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions,
                               token_slot, block_table, table_stride, page_size, tokens, nq, nkv, d,
                               rotary_half, interleaved, eps, write_cache, !tile_values, head0, row_width,
-                              v_head0, bias, stream);
+                              v_col0, dv, bias, stream);
         if (tile_values)
             hipLaunchKernelGGL(v_tile_write_kernel<bf16_t>, vgrid, block, 0, stream,
                                (const bf16_t*)qkv, (bf16_t*)v_cache, positions, token_slot,
-                               block_table, table_stride, page_size, tokens, nq, nkv, d, row_width, v_head0, bias);
+                               block_table, table_stride, page_size, tokens, nq, nkv, d, row_width, v_col0, dv, bias);
     } else {
         return RL_ERR_ARG;
     }

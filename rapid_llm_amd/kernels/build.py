@@ -12,6 +12,8 @@ Two kinds of library exist:
 * ``attn_d<D>``: the matrix-core attention kernels, compiled for one head size ``D``.
   A model compiles only the head sizes it has.
 * ``mlstm``: the matrix-memory recurrence, compiled when a model has such a mixer.
+* ``attn_tile_d<D>_v<DV>``: the tile attention for key heads of ``D`` and value heads of ``DV``
+  channels, compiled when a model has a mixer that needs it.
 
 There is no other implementation behind these: if ``hipcc`` is missing or a compile
 fails, loading raises.
@@ -44,11 +46,15 @@ CORE_SOURCES = (
 )
 ATTENTION_SOURCES = ("attention_mfma.hip", "attention_f32.hip")
 MLSTM_SOURCES = ("mlstm.hip",)
+ATTENTION_TILE_SOURCES = ("attention_tile.hip",)
 HEADERS = ("common.h", "static_entry.h")
 
 # head sizes built ahead of time by build_all(): every one the kernels take.  A fresh
 # checkout compiles only the head size of the model it is asked to run.
 DEFAULT_HEAD_DIMS = tuple(range(16, 257, 16))
+
+# pairs of (key, value) head sizes of the tile attention that build_all() builds ahead of time
+DEFAULT_TILE_HEAD_DIMS = ((16, 32), (32, 16), (64, 32), (64, 64), (128, 64), (128, 128))
 
 _HIPCC_FLAGS = (
     "-O3",
@@ -216,9 +222,18 @@ def mlstm_library(force: bool = False) -> Path:
     return compile_library("mlstm", MLSTM_SOURCES, force=force)
 
 
+def attention_tile_library(head_dim: int, value_dim: int, force: bool = False) -> Path:
+    for size in (head_dim, value_dim):
+        if size % 16 or not 16 <= size <= 256:
+            raise KernelBuildError(f"the tile attention takes head sizes in steps of 16 up to 256, got {size}")
+    flags = (f"-DRL_HEAD_DIM={head_dim}", f"-DRL_VALUE_DIM={value_dim}", "-mllvm", "-amdgpu-mfma-vgpr-form=1")
+    return compile_library(f"attn_tile_d{head_dim}_v{value_dim}", ATTENTION_TILE_SOURCES, flags, force=force)
+
+
 def build_all(head_dims: tuple[int, ...] = DEFAULT_HEAD_DIMS, force: bool = True) -> list[Path]:
     """Compile every library (what ``__graft_entry__.build`` calls)."""
     out = [core_library(force=force), mlstm_library(force=force)]
+    out += [attention_tile_library(d, dv, force=force) for d, dv in DEFAULT_TILE_HEAD_DIMS]
     if not all((CSRC / s).is_file() for s in ATTENTION_SOURCES):
         return out
     with ThreadPoolExecutor(min(8, len(head_dims))) as pool:

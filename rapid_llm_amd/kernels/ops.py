@@ -82,6 +82,19 @@ def attention_lib(head_dim: int) -> ctypes.CDLL:
     return lib
 
 
+_attn_tile: dict[tuple[int, int], ctypes.CDLL] = {}
+
+
+def attention_tile_lib(head_dim: int, value_dim: int) -> ctypes.CDLL:
+    lib = _attn_tile.get((head_dim, value_dim))
+    if lib is None:
+        lib = build.load(build.attention_tile_library(head_dim, value_dim))
+        if (lib.rl_attn_tile_head_dim(), lib.rl_attn_tile_value_dim()) != (head_dim, value_dim):
+            raise KernelError(f"tile attention library for head sizes {head_dim} / {value_dim} reports others")
+        _attn_tile[(head_dim, value_dim)] = lib
+    return lib
+
+
 def mlstm_lib() -> ctypes.CDLL:
     global _mlstm
     if _mlstm is None:
@@ -137,9 +150,12 @@ def _ok(code: int, what: str) -> None:
 
 
 def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, fed: Optional[torch.Tensor] = None,
-          scale: float = 1.0) -> None:
+          scale: float = 1.0, positions: Optional[torch.Tensor] = None,
+          inv_freq: Optional[torch.Tensor] = None) -> None:
     """``out[t] = table[ids[t]] * scale``; an id ``-(r + 1)`` takes ``fed[r]``, the token a
-    sampling kernel chose in row ``r`` of the previous step."""
+    sampling kernel chose in row ``r`` of the previous step.  With ``inv_freq`` (float32, one
+    frequency per pair of channels) the sinusoidal vector of ``positions[t]`` is added: channel
+    ``2i`` gets the sine, ``2i + 1`` the cosine of the float32 product ``positions[t] * inv_freq[i]``."""
     tokens = ids.numel()
     vocab, hidden = table.shape
     _need(ids, "ids", torch.int32)
@@ -147,10 +163,16 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, fed: Option
     _need(out, "out", torch.float32, (tokens, hidden))
     if fed is not None:
         _need(fed, "fed", torch.int32)
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", torch.float32, ((hidden + 1) // 2,))
+        if positions is None:
+            raise KernelError("a sinusoidal position vector needs the tokens' positions")
+        _need(positions, "positions", torch.int32, (tokens,))
     _ok(
         core().rl_embed(
             _p(ids), _p(fed), 0 if fed is None else fed.numel(), _p(table), _tag(table.dtype), _p(out),
-            tokens, hidden, vocab, ctypes.c_float(scale), _stream(),
+            tokens, hidden, vocab, ctypes.c_float(scale), _p(positions if inv_freq is not None else None),
+            _p(inv_freq), _stream(),
         ),
         "rl_embed",
     )
@@ -191,6 +213,88 @@ def add_rmsnorm(
         ),
         "rl_add_rmsnorm",
     )
+
+
+def normed_add_rmsnorm(
+    residual: torch.Tensor,
+    y: torch.Tensor,
+    y_weight: torch.Tensor,
+    y_eps: float,
+    weight: Optional[torch.Tensor],
+    out: Optional[torch.Tensor],
+    eps: float,
+    rows: Optional[torch.Tensor] = None,
+) -> None:
+    """``residual += rmsnorm(y) * y_weight`` (float32, in place), then, unless ``out`` is ``None``,
+    ``out = rmsnorm(residual) * weight``: a sub-layer's output that passes a norm of its own on
+    its way into the stream, and the next sub-layer's norm, in one kernel.  ``rows`` as in
+    :func:`add_rmsnorm`."""
+    tokens, hidden = residual.shape
+    _need(residual, "residual", torch.float32)
+    _need(y, "y", None, (tokens, hidden))
+    _need(y_weight, "norm weight of y", torch.float32, (hidden,))
+    out_rows = tokens if rows is None else rows.numel()
+    if out is not None:
+        _need(out, "out", y.dtype, (out_rows, hidden))
+        _need(weight, "norm weight", torch.float32, (hidden,))
+    if rows is not None:
+        _need(rows, "rows", torch.int32)
+    _ok(
+        core().rl_normed_add_rmsnorm(
+            _p(residual), _p(y), _p(y_weight), ctypes.c_float(y_eps), _p(weight if out is not None else None),
+            _p(out), _p(rows), out_rows, hidden, ctypes.c_float(eps), _tag(y.dtype), _stream(),
+        ),
+        "rl_normed_add_rmsnorm",
+    )
+
+
+def pair_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[t] = [a[t] | b[t]]``: two float32 streams side by side in ``out``'s type."""
+    tokens, hidden = a.shape
+    _need(a, "a", torch.float32)
+    _need(b, "b", torch.float32, (tokens, hidden))
+    _need(out, "out", None, (tokens, 2 * hidden))
+    _ok(core().rl_pair_rows(_p(a), _p(b), _p(out), tokens, hidden, _tag(out.dtype), _stream()), "rl_pair_rows")
+
+
+UNARY_ACTIVATIONS = {"gelu_tanh": 0, "relu_squared": 1}
+
+
+def unary_act(x: torch.Tensor, out: torch.Tensor, kind: str, route: Optional[torch.Tensor] = None,
+              expert_ff: int = 0) -> None:
+    """``out = act(x)`` for a one-operand activation (:data:`UNARY_ACTIVATIONS`).  With ``route``
+    (float32 ``[tokens, experts]``) the first ``experts * expert_ff`` columns are the hidden units
+    of the experts side by side and expert ``e``'s are multiplied by ``route[t, e]``."""
+    if kind not in UNARY_ACTIVATIONS:
+        raise KernelError(f"activation {kind!r} is not one of {sorted(UNARY_ACTIVATIONS)}")
+    tokens, cols = x.shape
+    _need(x, "x")
+    _need(out, "out", x.dtype, (tokens, cols))
+    experts = 0
+    if route is not None:
+        experts = route.shape[1]
+        _need(route, "route", torch.float32, (tokens, experts))
+        if expert_ff < 1 or experts * expert_ff > cols:
+            raise KernelError(f"{experts} experts of {expert_ff} hidden units do not fit rows of {cols}")
+    _ok(
+        core().rl_unary_act(_p(x), _p(out), tokens, cols, UNARY_ACTIVATIONS[kind], _p(route), experts, expert_ff,
+                            _tag(x.dtype), _stream()),
+        "rl_unary_act",
+    )
+
+
+ROUTE_MAX_EXPERTS = 1024
+
+
+def route(logits: torch.Tensor, top: int, scale: float) -> None:
+    """In place: router logits ``[tokens, experts]`` (float32) become the experts' weights: the
+    softmax scores of the ``top`` largest, divided by their sum (+ 1e-20), times ``scale``; 0
+    for every other expert."""
+    tokens, experts = logits.shape
+    _need(logits, "router logits", torch.float32)
+    if not 1 <= top <= experts <= ROUTE_MAX_EXPERTS:
+        raise KernelError(f"the router kernel chooses 1 to {experts} of at most {ROUTE_MAX_EXPERTS} experts, not {top}")
+    _ok(core().rl_route(_p(logits), tokens, experts, top, ctypes.c_float(scale), _stream()), "rl_route")
 
 
 GLU_ALPHA = 1.702  # the sigmoid's slope in the clamped gated activation
@@ -286,6 +390,7 @@ def qknorm_rope_kvwrite(
     pairing: str = "half_split",
     value_head0: Optional[int] = None,
     bias: Optional[torch.Tensor] = None,
+    value_dim: Optional[int] = None,
 ) -> None:
     """Norm + rotate q and k, write k and v to the cache pages (skipped when the caches
     are ``None``: a layer that reads another layer's cache).  ``q_out`` ``None``: the query
@@ -298,7 +403,8 @@ def qknorm_rope_kvwrite(
     A packed row holds the query heads, then the key heads, and the value heads from head
     ``value_head0`` on (default ``nq + nkv``, right behind the keys; ``nq``: the values are the
     keys as projected, before the rotation); it may be wider than that (columns of the same
-    product that another kernel reads).  ``bias`` (float32, one entry a column of the packed
+    product that another kernel reads).  ``value_dim``: the size of a value head where it is not
+    ``d`` (the values then lie behind the keys).  ``bias`` (float32, one entry a column of the packed
     row): the projection's bias, added to the heads as they are read, before norm and rotation,
     instead of by a kernel of its own after the product."""
     if pairing not in ROTARY_PAIRINGS:
@@ -306,13 +412,18 @@ def qknorm_rope_kvwrite(
     tokens = qkv.shape[0]
     if value_head0 is None:
         value_head0 = nq + nkv
+    dv = d if value_dim is None else int(value_dim)
+    if dv != d and value_head0 != nq + nkv:
+        raise KernelError("value heads of a size of their own lie behind the keys")
+    value_col0 = value_head0 * d
     _need(qkv, "qkv", None, (tokens, None))
     row_width = qkv.shape[1]
-    if value_head0 < 0 or row_width < (max(value_head0, nq) + nkv) * d or (d % 8 == 0 and row_width % 8):
+    if (value_head0 < 0 or not 1 <= dv <= 256 or row_width < max(value_col0 + nkv * dv, (nq + nkv) * d)
+            or (d % 8 == 0 and row_width % 8)):
         # (heads in steps of 8 channels are read 8 or 16 bytes at a time, so rows must start aligned)
         raise KernelError(
-            f"packed rows of {row_width} columns do not hold {nq} query, {nkv} key and {nkv} value heads "
-            f"of {d} (values from head {value_head0}) in whole groups of 8 columns"
+            f"packed rows of {row_width} columns do not hold {nq} query and {nkv} key heads of {d} and {nkv} "
+            f"value heads of {dv} (values from column {value_col0}) in whole groups of 8 columns"
         )
     if q_out is not None:
         _need(q_out, "q_out", qkv.dtype, (tokens, nq * d))
@@ -323,7 +434,7 @@ def qknorm_rope_kvwrite(
     if write:
         pages = k_cache.shape[0]
         _need(k_cache, "k_cache", qkv.dtype, (pages, nkv, page_size, d))
-        _need(v_cache, "v_cache", qkv.dtype, (pages, nkv, d, page_size))
+        _need(v_cache, "v_cache", qkv.dtype, (pages, nkv, dv, page_size))
         if max_position // page_size >= block_table.shape[1]:
             raise KernelError(
                 f"position {max_position} needs page {max_position // page_size} of a block "
@@ -350,7 +461,7 @@ def qknorm_rope_kvwrite(
             _p(qkv), _p(q_out), _p(k_cache), _p(v_cache), _p(q_norm_w), _p(k_norm_w), _p(cos),
             _p(sin), _p(positions), _p(token_slot), _p(block_table), block_table.stride(0),
             page_size, tokens, nq, nkv, d, half, ROTARY_PAIRINGS[pairing], ctypes.c_float(eps), int(write),
-            row_width, value_head0, _p(bias), _tag(qkv.dtype), _stream(),
+            row_width, value_col0, dv, _p(bias), _tag(qkv.dtype), _stream(),
         ),
         "rl_qknorm_rope_kvwrite",
     )
@@ -371,13 +482,17 @@ def attention_generic(
     window: int,
     scale: float,
     max_position: int,
+    value_dim: Optional[int] = None,
+    keep_first: int = 0,
+    sink: bool = False,
 ) -> None:
     tokens = q.shape[0]
     pages = k_cache.shape[0]
+    dv = d if value_dim is None else int(value_dim)
     _need(q, "q", None, (tokens, nq * d))
-    _need(out, "out", q.dtype, (tokens, nq * d))
+    _need(out, "out", q.dtype, (tokens, nq * dv))
     _need(k_cache, "k_cache", q.dtype, (pages, nkv, page_size, d))
-    _need(v_cache, "v_cache", q.dtype, (pages, nkv, d, page_size))
+    _need(v_cache, "v_cache", q.dtype, (pages, nkv, dv, page_size))
     _need(positions, "positions", torch.int32, (tokens,))
     _need(token_slot, "token_slot", torch.int32, (tokens,))
     _need(block_table, "block_table", torch.int32)
@@ -390,7 +505,7 @@ def attention_generic(
         core().rl_attention_generic(
             _p(q), _p(k_cache), _p(v_cache), _p(out), _p(positions), _p(token_slot),
             _p(block_table), block_table.stride(0), page_size, tokens, nq, nkv, d, window,
-            ctypes.c_float(scale), _tag(q.dtype), _stream(),
+            ctypes.c_float(scale), dv, int(keep_first), int(bool(sink)), _tag(q.dtype), _stream(),
         ),
         "rl_attention_generic",
     )
@@ -1094,6 +1209,56 @@ def attention_f32(
     )
 
 
+def attention_tile(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    out: torch.Tensor,
+    ctx,
+    block_table: torch.Tensor,
+    page_size: int,
+    nq: int,
+    nkv: int,
+    d: int,
+    dv: int,
+    window: int,
+    keep_first: int,
+    sink: bool,
+    scale: float,
+) -> None:
+    """Attention of every token of the step, in tiles of 16 rows on the matrix cores, for value
+    heads of a size of their own, a window that keeps a request's first ``keep_first`` positions
+    visible, and (``sink``) a softmax with 1 added to its denominator.  float32 (bit for bit the
+    same however the step was cut) or bfloat16."""
+    tokens = q.shape[0]
+    pages = k_cache.shape[0]
+    _need(q, "q", None, (tokens, nq * d))
+    _need(out, "out", q.dtype, (tokens, nq * dv))
+    _need(k_cache, "k_cache", q.dtype, (pages, nkv, page_size, d))
+    _need(v_cache, "v_cache", q.dtype, (pages, nkv, dv, page_size))
+    _need(ctx.positions, "positions", torch.int32, (tokens,))
+    _need(ctx.token_slot, "token_slot", torch.int32, (tokens,))
+    _need(block_table, "block_table", torch.int32)
+    if page_size % 4:
+        raise KernelError(f"the tile attention reads four keys of a page at once: page size {page_size}")
+    if ctx.max_position // page_size >= block_table.shape[1]:
+        raise KernelError(
+            f"position {ctx.max_position} needs page {ctx.max_position // page_size} of a block table "
+            f"with {block_table.shape[1]} columns"
+        )
+    if nkv > 65535 or window < 0 or keep_first < 0:
+        raise KernelError(f"{nkv} kv heads, window {window}, {keep_first} kept positions")
+    tiles, num_tiles = _f32_tiles(ctx, nq // nkv)
+    _ok(
+        attention_tile_lib(d, dv).rl_attn_tile(
+            _p(q), _p(k_cache), _p(v_cache), _p(out), _p(tiles), num_tiles, _p(ctx.positions),
+            _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv, window,
+            int(keep_first), int(bool(sink)), ctypes.c_float(scale), _tag(q.dtype), _stream(),
+        ),
+        "rl_attn_tile",
+    )
+
+
 def paged_attention(
     q: torch.Tensor,
     k_cache: torch.Tensor,
@@ -1108,6 +1273,9 @@ def paged_attention(
     window: int,
     scale: float,
     prepare: Optional[tuple] = None,
+    value_dim: Optional[int] = None,
+    keep_first: int = 0,
+    sink: bool = False,
 ) -> None:
     """Attention of every token of the step over its request's cached keys.
 
@@ -1117,9 +1285,29 @@ def paged_attention(
 
     ``prepare`` = ``(q_norm_w, cos, sin, eps)``: ``q`` is the packed [q | k | v] row of every token,
     and the kernels norm and rotate the query heads as they read them (only where
-    :func:`attention_prepares_queries` says so)."""
+    :func:`attention_prepares_queries` says so).
+
+    ``value_dim`` (the size of a value head, where it is not ``d``), ``keep_first`` (with a window:
+    the request's first positions stay visible behind it) and ``sink`` (1 added to the softmax's
+    denominator: a key of score 0 without a value) send the step to the kernels that take them:
+    tiles of 16 rows on the matrix cores for head sizes in steps of 16, the FMA kernel otherwise."""
     if prepare is not None and not attention_prepares_queries(q.dtype, d, 0 if prepare[1] is None else prepare[1].shape[1]):
         raise KernelError("the attention kernels do not finish the queries of this head size, type or rotation")
+    dv = d if value_dim is None else int(value_dim)
+    keep_first = int(keep_first) if window > 0 else 0  # without a window every key is seen anyway
+    if dv != d or keep_first or sink:
+        # value heads of their own size, kept first positions, one more term in the denominator
+        if prepare is not None:
+            raise KernelError("queries are finished before an attention with these options")
+        if d % 16 == 0 and dv % 16 == 0 and page_size % 4 == 0:
+            attention_tile(q, k_cache, v_cache, out, ctx, block_table, page_size, nq, nkv, d, dv,
+                           window, keep_first, sink, scale)
+        else:
+            attention_generic(
+                q, k_cache, v_cache, out, ctx.positions, ctx.token_slot, block_table, page_size,
+                nq, nkv, d, window, scale, ctx.max_position, dv, keep_first, sink,
+            )
+        return
     if q.dtype == torch.float32 and d % 16 == 0:
         attention_f32(q, k_cache, v_cache, out, ctx, block_table, page_size, nq, nkv, d, window, scale)
         return

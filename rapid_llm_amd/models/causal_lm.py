@@ -23,7 +23,8 @@ from ..parts.base import (
     CacheNeed,
     ParamSpec,
 )
-from ..parts.lazy import plain, run_norm
+from ..parts.inject import StreamMix
+from ..parts.lazy import plain, run_norm, settle
 from ..parts.offsets import StreamOffsetTable
 from .spec import ModelSpec
 
@@ -47,6 +48,13 @@ class CausalLM:
                 if not 0 <= place < len(self.order):
                     raise ValueError(f"a stream offset names place {place} of a run order of {len(self.order)}")
             self.offsets = StreamOffsetTable(so.checkpoint_name, so.places, spec.hidden_size, name="stream_offsets")
+        self.mixes = None
+        if spec.stream_mixes is not None:
+            sm = spec.stream_mixes
+            for place in sm.places:
+                if not 0 <= place < len(self.order):
+                    raise ValueError(f"a stream mix names place {place} of a run order of {len(self.order)}")
+            self.mixes = StreamMix(sm.checkpoint_name, sm.places, spec.hidden_size, name="stream_mix")
         self._positions: dict[str, object] = {}
         self.blocks = []
         for i, layer in enumerate(spec.layers):
@@ -69,6 +77,18 @@ class CausalLM:
                     layer.feed_forward_norm.kind, **layer.feed_forward_norm.params, name=f"layers.{i}.ff_norm"
                 )
             n1 = NORMS.create(layer.mixer_norm.kind, **layer.mixer_norm.params, name=f"layers.{i}.mixer_norm")
+            post = {}
+            if layer.mixer_post_norm is not None:
+                post["mixer_post_norm"] = NORMS.create(
+                    layer.mixer_post_norm.kind, **layer.mixer_post_norm.params, name=f"layers.{i}.mixer_post_norm"
+                )
+            if layer.feed_forward_post_norm is not None:
+                if ff is None:
+                    raise ValueError(f"layer {i}: a norm behind a feed-forward that is not there")
+                post["feed_forward_post_norm"] = NORMS.create(
+                    layer.feed_forward_post_norm.kind, **layer.feed_forward_post_norm.params,
+                    name=f"layers.{i}.ff_post_norm",
+                )
             self.blocks.append(
                 BLOCKS.create(
                     layer.block.kind,
@@ -77,6 +97,7 @@ class CausalLM:
                     feed_forward=ff,
                     mixer_norm=n1,
                     feed_forward_norm=n2,
+                    **post,
                 )
             )
 
@@ -89,6 +110,8 @@ class CausalLM:
         yield self.output
         if self.offsets is not None:
             yield self.offsets
+        if self.mixes is not None:
+            yield self.mixes
         yield from self._positions.values()
 
     def param_specs(self) -> list[ParamSpec]:
@@ -133,13 +156,22 @@ class CausalLM:
         """Run the tokens of ``ctx`` through every layer (which writes their keys and values)
         and return float32 logits ``[len(ctx.logit_rows), vocab]``."""
         residual = self.embed.forward(ctx.token_ids, ctx)
+        # the embedding's output, which the stream mixes take in again (the stream itself is
+        # updated in place)
+        first = residual.clone() if self.mixes is not None else None
         delta = None
         for place, li in enumerate(self.order):
             block = self.blocks[li]
+            if self.mixes is not None and self.mixes.at(place):
+                delta = settle(residual, delta)
+                if delta is not None:
+                    residual.add_(delta)
+                    delta = None
+                residual = self.mixes.forward(residual, first)
             if self.offsets is not None:
                 self.offsets.add(residual, place)
             if not getattr(block, "accepts_deferred", False):
-                delta = plain(delta)
+                delta = settle(residual, delta)
             delta = block.forward(residual, delta, ctx, caches[place])
         if ctx.num_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=residual.device)

@@ -20,6 +20,14 @@ projection, a token's values are its keys as projected, before the rotation; the
 projection of one number per query head rides in the same product (rows behind the keys and
 values, padded to a multiple of 8), and every head's output is multiplied by the sigmoid of its
 number before the output projection.
+
+Three more options send a layer to the attention kernels that take them (tiles of 16 rows on the
+matrix cores, in both types).  ``value_dim``: value heads of a size of their own (the packed row
+is ``[q | k | v]`` with narrower or wider ``v`` heads, the value pages and the heads' outputs have
+that size, the output projection reads ``num_heads * value_dim`` columns).  ``keep_first``: with
+a window, a request's first positions stay visible to every later query, and their pages stay
+mapped.  ``sink``: the softmax's denominator is ``1 + sum_j exp(s_j)``, as if one more key of
+score 0 and without a value were always seen.
 """
 
 from __future__ import annotations
@@ -59,6 +67,9 @@ class GQAAttention(Mixer):
         values: str = "own",
         head_gate_name: str | None = None,
         bias_names: dict[str, str] | None = None,
+        value_dim: int | None = None,
+        keep_first: int = 0,
+        sink: bool = False,
     ) -> None:
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not divisible by {num_kv_heads} kv heads")
@@ -68,6 +79,15 @@ class GQAAttention(Mixer):
             raise ValueError(f"attention kernels take even head sizes up to 256, got {head_dim}")
         self.hidden_size = hidden_size
         self.nq, self.nkv, self.d = num_heads, num_kv_heads, head_dim
+        self.dv = head_dim if value_dim is None else int(value_dim)
+        if not 1 <= self.dv <= 256:
+            raise ValueError(f"attention kernels take value heads of up to 256 channels, got {self.dv}")
+        if self.dv != head_dim and (values == "keys" or head_gate_name):
+            raise ValueError("value heads of a size of their own come with a value projection and without head gates")
+        if keep_first < 0:
+            raise ValueError(f"a window keeps a number of first positions, not {keep_first}")
+        self.keep_first = int(keep_first) if window else 0  # without a window every key is seen
+        self.sink = bool(sink)
         self.prefix = checkpoint_prefix
         self.qk_norm_eps = qk_norm_eps
         self.window = int(window)
@@ -92,12 +112,15 @@ class GQAAttention(Mixer):
         # the packed row: query heads, key heads, value heads unless they are the keys, then
         # one gate per query head, padded so that rows stay whole groups of 8 columns
         self.value_head0 = num_heads if self.values_are_keys else num_heads + num_kv_heads
-        self.qkv_rows = (num_heads + (1 if self.values_are_keys else 2) * num_kv_heads) * head_dim
+        self.qkv_rows = (num_heads + num_kv_heads) * head_dim + (0 if self.values_are_keys else num_kv_heads * self.dv)
         self.gate_rows = num_heads if head_gate_name else 0
         self.gate_pad = -(self.qkv_rows + self.gate_rows) % 8 if self.gate_rows else 0
-        self.plain_row = not self.values_are_keys and not self.gate_rows
-        self.qkv = Linear(hidden_size, self.qkv_rows + self.gate_rows + self.gate_pad)
-        self.o = Linear(num_heads * head_dim, hidden_size)
+        # the options that only the tile kernels (or the kernel for any size) take
+        self.extended = self.dv != head_dim or self.keep_first > 0 or self.sink
+        self.plain_row = not self.values_are_keys and not self.gate_rows and not self.extended
+        self.row_pad = -self.qkv_rows % 8 if (self.extended and not self.gate_rows) else 0
+        self.qkv = Linear(hidden_size, self.qkv_rows + self.gate_rows + self.gate_pad + self.row_pad)
+        self.o = Linear(num_heads * self.dv, hidden_size)
         self.q_norm_w = self.k_norm_w = None
         # Qwen3 has neither (rapid_llm/models/qwen3.py:16-18: qkv_bias=False); architectures of the
         # same skeleton do (rapid_llm/models/base.py:121-132 passes bias=qkv_bias), under the
@@ -108,16 +131,18 @@ class GQAAttention(Mixer):
     def param_specs(self) -> list[ParamSpec]:
         p, n = self.prefix, self.names
         q_rows, kv_rows = self.nq * self.d, self.nkv * self.d
+        v_rows = self.nkv * self.dv
         packed = [Source(p + n["q"], q_rows), Source(p + n["k"], kv_rows)]
         if not self.values_are_keys:
-            packed.append(Source(p + n["v"], kv_rows))
+            packed.append(Source(p + n["v"], v_rows))
         if self.gate_rows:
             packed.append(Source(p + n["g"], self.gate_rows))
-        if self.gate_pad:
-            packed.append(Source("", self.gate_pad))  # rows of zeros
+        if self.gate_pad + self.row_pad:
+            packed.append(Source("", self.gate_pad + self.row_pad))  # rows of zeros
         specs = [
             ParamSpec(self.name + ".qkv", (self.qkv.out_features, self.hidden_size), "matrix", tuple(packed)),
-            ParamSpec(self.name + ".o", (self.hidden_size, q_rows), "matrix", (Source(p + n["o"], self.hidden_size),)),
+            ParamSpec(self.name + ".o", (self.hidden_size, self.nq * self.dv), "matrix",
+                      (Source(p + n["o"], self.hidden_size),)),
         ]
         if self.qk_norm_eps is not None:
             specs += [
@@ -134,9 +159,9 @@ class GQAAttention(Mixer):
         if self.qkv_bias:
             biases = [Source(p + bias_of("q"), q_rows), Source(p + bias_of("k"), kv_rows)]
             if not self.values_are_keys:
-                biases.append(Source(p + bias_of("v"), kv_rows))
-            if self.gate_rows + self.gate_pad:
-                biases.append(Source("", self.gate_rows + self.gate_pad))  # the gates have none
+                biases.append(Source(p + bias_of("v"), v_rows))
+            if self.gate_rows + self.gate_pad + self.row_pad:
+                biases.append(Source("", self.gate_rows + self.gate_pad + self.row_pad))  # the gates have none
             specs.append(ParamSpec(self.name + ".qkv_bias", (self.qkv.out_features,), "vector", tuple(biases)))
         if self.o_bias:
             specs.append(ParamSpec(
@@ -160,9 +185,13 @@ class GQAAttention(Mixer):
 
     # ---- cache -----------------------------------------------------------------
     def cache_need(self) -> CacheNeed:
-        return CacheNeed.keys_and_values(self.nkv, self.d, window=self.window)
+        return CacheNeed.keys_and_values(
+            self.nkv, self.d, window=self.window, value_dim=self.dv, keep_first=self.keep_first
+        )
 
     def recorded_step_bytes(self, rows: int, context_bound: int, page_size: int) -> int:
+        if self.extended:
+            return 0  # one kernel, nothing kept between two
         return ops.decode_scratch_bytes(rows, self.nq, self.nkv, self.d, context_bound, page_size, self.window)
 
     # ---- step ------------------------------------------------------------------
@@ -178,7 +207,7 @@ class GQAAttention(Mixer):
         cos = pos_enc.cos if pos_enc is not None else None
         sin = pos_enc.sin if pos_enc is not None else None
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
-        out = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
+        out = torch.empty((tokens, self.nq * self.dv), dtype=qkv.dtype, device=x.device)
         rotary_half = cos.shape[1] if cos is not None else 0
         pairing = getattr(pos_enc, "pairing", "half_split") if cos is not None else "half_split"
         if self.plain_row and ops.decode_attention_fusable(
@@ -201,11 +230,13 @@ class GQAAttention(Mixer):
             self.q_norm_w, self.k_norm_w, cos, sin,
             ctx.positions, ctx.token_slot, table, cache.page_size,
             self.nq, self.nkv, self.d, eps, ctx.max_position, pairing, self.value_head0, self.bias_in_kernel,
+            self.dv,
         )
         ops.paged_attention(
             qkv if in_kernel else q, cache.k, cache.v, out, ctx, table, cache.page_size,
             self.nq, self.nkv, self.d, self.window, self.scale,
             prepare=(self.q_norm_w, cos, sin, eps) if in_kernel else None,
+            value_dim=self.dv, keep_first=self.keep_first, sink=self.sink,
         )
         if self.gate_rows:
             ops.head_gate(out, qkv, self.qkv_rows, self.nq, self.d)

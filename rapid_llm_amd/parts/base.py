@@ -38,7 +38,8 @@ if TYPE_CHECKING:  # pragma: no cover
 
 @dataclass(frozen=True)
 class Source:
-    """One checkpoint tensor feeding ``rows`` rows (dim 0) of a parameter.  An empty name
+    """One checkpoint tensor feeding ``rows`` rows of a parameter (dim 0, or the parameter's
+    ``axis``).  An empty name
     stands for ``rows`` rows of zeros that no checkpoint tensor feeds (padding of a packed
     matrix to a width its kernels take)."""
 
@@ -52,7 +53,9 @@ class ParamSpec:
 
     ``sources`` are concatenated along dim 0 in order: a fused matrix such as the packed
     query/key/value projection lists its three checkpoint tensors
-    (rapid_llm/modules/linear.py:253-271 writes the same row blocks).
+    (rapid_llm/modules/linear.py:253-271 writes the same row blocks).  ``axis`` 1 lays them side
+    by side instead (matrices ``[out, in_i]`` that share their output and are applied to the
+    concatenation of their inputs: the down projections of several experts).
 
     ``role`` decides the storage type:
       * ``"matrix"``: the engine's compute type; in a bfloat16 engine a tensor the
@@ -73,6 +76,11 @@ class ParamSpec:
     sources: tuple[Source, ...]
     init: str = "normal"  # "normal" | "norm" | "zeros" | "table"
     fallback: str | None = None
+    axis: int = 0
+
+    def source_shape(self, rows: int) -> tuple[int, ...]:
+        """Shape of a checkpoint tensor that feeds ``rows`` of this parameter's ``axis``."""
+        return (*self.shape[: self.axis], rows, *self.shape[self.axis + 1 :])
 
 
 @dataclass(frozen=True)
@@ -127,7 +135,8 @@ class CacheNeed:
     ``kind == "paged"``: tensors that grow with the request, in pages, each named and laid out
     by a :class:`PagedSpec` (keys and values here; a mixer may name one latent row, or keys and
     values of different widths).  ``window`` 0 keeps every position, otherwise only the last
-    ``window`` positions of a request are kept and older pages are given back.
+    ``window`` positions of a request are kept and older pages are given back, except the pages
+    of the first ``keep_first`` positions, which every later query still reads.
     ``kind == "state"``: nothing paged.  Fixed-size per-request tensors the mixer owns, zeroed
     when a request takes the slot, may accompany either kind: one as ``state_shape`` (and
     ``state_dtype``), or several, each under a name, as ``states`` (a mixer with a short
@@ -138,6 +147,7 @@ class CacheNeed:
 
     kind: str  # "paged" | "state" | "none"
     window: int = 0
+    keep_first: int = 0  # with a window: the first positions of a request that stay readable
     paged: tuple[PagedSpec, ...] = ()
     state_shape: tuple[int, ...] | None = None
     state_dtype: str | None = None  # torch dtype name; None: the engine's compute type
@@ -147,6 +157,8 @@ class CacheNeed:
     def __post_init__(self) -> None:
         if self.kind not in ("paged", "state", "none"):
             raise ValueError(f"a cache need is 'paged', 'state' or 'none', not {self.kind!r}")
+        if self.keep_first < 0 or self.window < 0:
+            raise ValueError(f"a window of {self.window} with {self.keep_first} kept first positions")
         if (self.kind == "paged") != bool(self.paged):
             raise ValueError(f"a {self.kind!r} cache need names {len(self.paged)} paged tensors")
         names = [p.name for p in self.paged]
@@ -154,12 +166,14 @@ class CacheNeed:
             raise ValueError(f"a mixer names two paged tensors alike: {names}")
 
     @classmethod
-    def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int = 0, **more) -> "CacheNeed":
+    def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int = 0, value_dim: int | None = None,
+                        **more) -> "CacheNeed":
         """The layout the attention kernels of this package read: keys ``[pages, heads,
-        page_size, head_dim]`` under ``"k"``, values transposed ``[pages, heads, head_dim,
-        page_size]`` under ``"v"``."""
+        page_size, head_dim]`` under ``"k"``, values transposed ``[pages, heads, value_dim,
+        page_size]`` under ``"v"`` (``value_dim`` defaults to ``head_dim``)."""
         shape = (num_kv_heads, head_dim)
-        return cls("paged", window=window, paged=(PagedSpec("k", shape, 1), PagedSpec("v", shape, 2)), **more)
+        vshape = (num_kv_heads, head_dim if value_dim is None else value_dim)
+        return cls("paged", window=window, paged=(PagedSpec("k", shape, 1), PagedSpec("v", vshape, 2)), **more)
 
     def state_specs(self) -> tuple[StateSpec, ...]:
         """Every per-request tensor asked for; the one given as ``state_shape`` is named ``"state"``."""

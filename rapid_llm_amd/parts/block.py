@@ -1,5 +1,6 @@
 """Pre-norm arrangement: ``r += mixer(norm(r)); r += feed_forward(norm(r))``; a layer
-without a feed-forward has the first sub-layer only.
+without a feed-forward has the first sub-layer only.  The sandwich arrangement has a second
+norm behind each sub-layer, applied to its output before the add.
 
 The add of each sub-layer's output is carried forward as ``delta`` and happens inside the
 next norm kernel, as the reference threads ``(hidden, residual)`` through its layers
@@ -9,7 +10,7 @@ next norm kernel, as the reference threads ``(hidden, residual)`` through its la
 from __future__ import annotations
 
 from .base import BLOCKS, Block
-from .lazy import run_norm
+from .lazy import NormedDelta, plain, run_norm
 
 
 class PreNormBlock(Block):
@@ -36,4 +37,44 @@ class PreNormBlock(Block):
         return self.feed_forward.forward(x, ctx)
 
 
+class SandwichBlock(Block):
+    """A norm before and after each sub-layer: ``r += post1(mixer(pre1(r)))``, then
+    ``r += post2(feed_forward(pre2(r)))``.  A sub-layer's output travels on as a
+    :class:`~rapid_llm_amd.parts.lazy.NormedDelta`: the norm that runs next applies the pending
+    post-norm, adds the result to the stream and computes its own rows in one kernel."""
+
+    replayable = True
+    accepts_deferred = True
+
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm, mixer_post_norm,
+                 feed_forward_post_norm=None) -> None:
+        if (feed_forward is None) != (feed_forward_post_norm is None):
+            raise ValueError("a feed-forward and the norm behind it come together or not at all")
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.feed_forward_norm = feed_forward_norm
+        self.mixer_post_norm = mixer_post_norm
+        self.feed_forward_post_norm = feed_forward_post_norm
+
+    def parts(self):
+        if self.feed_forward is None:
+            return (self.mixer_norm, self.mixer, self.mixer_post_norm)
+        return (self.mixer_norm, self.mixer, self.mixer_post_norm,
+                self.feed_forward_norm, self.feed_forward, self.feed_forward_post_norm)
+
+    @staticmethod
+    def _pending(norm, y):
+        return NormedDelta(plain(y), norm.weight, norm.eps)
+
+    def forward(self, residual, delta, ctx, cache):
+        x = run_norm(self.mixer_norm, residual, delta, ctx)
+        a = self._pending(self.mixer_post_norm, self.mixer.forward(x, ctx, cache))
+        if self.feed_forward is None:
+            return a
+        x = run_norm(self.feed_forward_norm, residual, a, ctx)
+        return self._pending(self.feed_forward_post_norm, self.feed_forward.forward(x, ctx))
+
+
 BLOCKS.register("prenorm", PreNormBlock)
+BLOCKS.register("sandwich", SandwichBlock)

@@ -18,9 +18,15 @@ class TokenEmbedding(Embedding):
     replayable = True
 
     def __init__(self, vocab_size: int, hidden_size: int, checkpoint_name: str, name: str = "embed",
-                 scale: float = 1.0) -> None:
+                 scale: float = 1.0, sinusoid_base: float | None = None) -> None:
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
         self.scale = float(scale)  # every row is multiplied by it on its way into the stream
+        # with a base b, the sinusoidal vector of the token's position p is added: channel 2i
+        # gets sin(p * b^(-2i/hidden)), channel 2i + 1 the cosine of the same angle
+        self.sinusoid_base = None if sinusoid_base is None else float(sinusoid_base)
+        if self.sinusoid_base is not None and not self.sinusoid_base > 0:
+            raise ValueError(f"the base of a sinusoidal position vector must be positive, got {sinusoid_base}")
+        self.inv_freq: torch.Tensor | None = None
         self.checkpoint_name = checkpoint_name
         self.name = name
         self.table: torch.Tensor | None = None
@@ -37,11 +43,16 @@ class TokenEmbedding(Embedding):
 
     def bind(self, params, runtime) -> None:
         self.table = params[self.name + ".weight"]
+        if self.sinusoid_base is not None:
+            i = torch.arange((self.hidden_size + 1) // 2, dtype=torch.float64)
+            inv = self.sinusoid_base ** (-2.0 * i / self.hidden_size)
+            self.inv_freq = inv.to(torch.float32).to(runtime.device)
 
     def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
         """Rows of the table for the ids; an id ``-(r + 1)`` takes ``ctx.fed_tokens[r]``."""
         out = torch.empty((token_ids.numel(), self.hidden_size), dtype=torch.float32, device=token_ids.device)
-        ops.embed(token_ids, self.table, out, getattr(ctx, "fed_tokens", None), self.scale)
+        ops.embed(token_ids, self.table, out, getattr(ctx, "fed_tokens", None), self.scale,
+                  ctx.positions if self.inv_freq is not None else None, self.inv_freq)
         return out
 
 

@@ -13,6 +13,12 @@ products on either side absorb it, without any part knowing its neighbours:
   of squares; the factor ``rsqrt(mean + eps)`` is a scalar per row and commutes with the
   consumer's own product, which applies it to its result.
 
+* :class:`NormedDelta`: what a block whose sub-layers pass a norm of their own on their way into
+  the stream returns in place of that norm's result: the sub-layer's output as it is, with the
+  norm's weight and epsilon.  A norm that declares ``fuses_products`` applies it, adds the result
+  to the stream and computes its own rows in one kernel; anything else gets the normed rows in
+  the stream's type from ``materialize()``.
+
 Blocks and models route these only between parts that declare them (``fuses_products`` on
 a norm, ``accepts_scaled_rows`` on a mixer or feed-forward, ``accepts_deferred`` on a
 block); everything else sees plain tensors.
@@ -39,6 +45,31 @@ class DeferredProduct:
         return self.linear(self.x, out_dtype)
 
 
+class NormedDelta:
+    """``rmsnorm(y) * weight``, not yet computed."""
+
+    def __init__(self, y: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+        self.y = y
+        self.weight = weight
+        self.eps = float(eps)
+
+    @property
+    def shape(self):
+        return self.y.shape
+
+    def add_to(self, residual: torch.Tensor) -> None:
+        """``residual += rmsnorm(y) * weight`` in place (float32)."""
+        from ..kernels import ops
+
+        ops.normed_add_rmsnorm(residual, self.y, self.weight, self.eps, None, None, 0.0)
+
+    def materialize(self, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        """The normed rows as a float32 tensor (what is added to the stream)."""
+        out = torch.zeros(self.y.shape, dtype=torch.float32, device=self.y.device)
+        self.add_to(out)
+        return out
+
+
 @dataclass
 class ScaledRows:
     rows: torch.Tensor  # [M, size], the residual rows times the norm's weight
@@ -61,7 +92,16 @@ class ScaledRows:
 
 def plain(value):
     """A tensor, whatever lazy value it still was."""
-    return value.materialize() if isinstance(value, DeferredProduct) else value
+    return value.materialize() if isinstance(value, (DeferredProduct, NormedDelta)) else value
+
+
+def settle(residual, delta):
+    """What is left to add once lazy values are settled: a pending normed delta joins the stream
+    now, a deferred product becomes a tensor."""
+    if isinstance(delta, NormedDelta):
+        delta.add_to(residual)
+        return None
+    return plain(delta)
 
 
 def run_norm(norm, residual, delta, ctx, consumer=None, rows=None):
@@ -70,4 +110,8 @@ def run_norm(norm, residual, delta, ctx, consumer=None, rows=None):
         return norm.forward(
             residual, delta, ctx, rows, scaled_ok=bool(getattr(consumer, "accepts_scaled_rows", False))
         )
+    if isinstance(delta, NormedDelta):
+        # a norm that knows nothing of it: the stream takes it first
+        delta.add_to(residual)
+        delta = None
     return norm.forward(residual, plain(delta), ctx, rows)

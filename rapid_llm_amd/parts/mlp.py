@@ -1,10 +1,13 @@
-"""Dense gated feed-forward: ``down(act(gate(x), up(x)))`` with ``act(g, u) = silu(g) * u``
+"""Feed-forwards.  Dense gated feed-forward: ``down(act(gate(x), up(x)))`` with ``act(g, u) = silu(g) * u``
 (SwiGLU), or, with a ``limit``, the clamped variant ``g' * sigmoid(alpha * g') * (u' + 1)`` where
 ``g' = min(g, limit)`` and ``u' = clamp(u, -limit, limit)``.
 
 Gate and up are one packed matrix ``[2I, H]`` with rows ``[gate | up]``
 (rapid_llm/models/base.py:401-404, rapid_llm/modules/linear.py:157-172), so one product
 feeds the activation kernel (rapid_llm/modules/mlp.py:67-68).
+
+Beside it a two-layer feed-forward without a gate, ``down(act(up(x)))``, and a mixture of such
+experts behind a softmax router.
 """
 
 from __future__ import annotations
@@ -74,5 +77,127 @@ class SwiGLU(FeedForward):
         return self.down.deferred(act, ctx)
 
 
+class TwoLayer(FeedForward):
+    """``down(act(up(x)))`` with a one-operand activation (``ops.UNARY_ACTIVATIONS``: the tanh form
+    of gelu, or the square of relu); no gate, no biases."""
+
+    replayable = True
+
+    def __init__(
+        self,
+        hidden_size: int,
+        intermediate_size: int,
+        checkpoint_prefix: str,
+        activation: str,
+        name: str = "ff",
+        up_name: str = "up",
+        down_name: str = "down",
+    ) -> None:
+        if activation not in ops.UNARY_ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not one of {sorted(ops.UNARY_ACTIVATIONS)}")
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.prefix, self.activation, self.name = checkpoint_prefix, activation, name
+        self.names = (up_name, down_name)
+        self.up = Linear(hidden_size, intermediate_size)
+        self.down = Linear(intermediate_size, hidden_size)
+
+    def param_specs(self) -> list[ParamSpec]:
+        h, i = self.hidden_size, self.intermediate_size
+        u, d = (self.prefix + n for n in self.names)
+        return [
+            ParamSpec(self.name + ".up", (i, h), "matrix", (Source(u, i),)),
+            ParamSpec(self.name + ".down", (h, i), "matrix", (Source(d, h),)),
+        ]
+
+    def bind(self, params, runtime) -> None:
+        self.up.bind(params[self.name + ".up"])
+        self.down.bind(params[self.name + ".down"])
+
+    def forward(self, x, ctx):
+        hidden = self.up(x)
+        ops.unary_act(hidden, hidden, self.activation)
+        return self.down.deferred(hidden, ctx)
+
+
+class RoutedExperts(FeedForward):
+    """A mixture of two-layer experts: every token uses the ``top`` experts that a softmax router
+    scores highest, weighted by their scores over the chosen ones' sum, times ``route_scale``;
+    a shared expert (``shared_size`` > 0) runs for every token and is added.
+
+    The router's product and scores are float32 in every engine (its matrix is held in
+    float32).  The experts' up projections are one packed matrix ``[experts * expert_size +
+    shared_size, hidden]`` and their down projections one matrix side by side over the same
+    columns, so a step is two products whatever the tokens chose: the activation kernel
+    multiplies every expert's hidden units by the token's weight for that expert, which is 0
+    for an expert the token does not use.  Every expert's weights are read in every step; nothing
+    is gathered, no shape depends on the routing, and a token's result does not depend on the
+    rest of the batch."""
+
+    replayable = True
+
+    def __init__(
+        self,
+        hidden_size: int,
+        num_experts: int,
+        top: int,
+        expert_size: int,
+        checkpoint_prefix: str,
+        activation: str,
+        route_scale: float = 1.0,
+        shared_size: int = 0,
+        name: str = "ff",
+        router_name: str = "router",
+        expert_prefix: str = "e",
+        shared_prefix: str = "shared.",
+        up_name: str = "up",
+        down_name: str = "down",
+    ) -> None:
+        if activation not in ops.UNARY_ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not one of {sorted(ops.UNARY_ACTIVATIONS)}")
+        if not 1 <= top <= num_experts <= ops.ROUTE_MAX_EXPERTS:
+            raise ValueError(f"a token uses 1 to {num_experts} of at most {ops.ROUTE_MAX_EXPERTS} experts, not {top}")
+        self.hidden_size, self.num_experts, self.top = hidden_size, num_experts, top
+        self.expert_size, self.shared_size = expert_size, shared_size
+        self.route_scale = float(route_scale)
+        self.prefix, self.activation, self.name = checkpoint_prefix, activation, name
+        self.names = (router_name, expert_prefix, shared_prefix, up_name, down_name)
+        self.inner = num_experts * expert_size + shared_size
+        self.router = Linear(hidden_size, num_experts)
+        self.up = Linear(hidden_size, self.inner)
+        self.down = Linear(self.inner, hidden_size)
+
+    def _sources(self, which: str, rows_of_expert: int, rows_of_shared: int) -> tuple[Source, ...]:
+        _, expert, shared, _, _ = self.names
+        out = [Source(f"{self.prefix}{expert}{e}.{which}", rows_of_expert) for e in range(self.num_experts)]
+        if self.shared_size:
+            out.append(Source(f"{self.prefix}{shared}{which}", rows_of_shared))
+        return tuple(out)
+
+    def param_specs(self) -> list[ParamSpec]:
+        h = self.hidden_size
+        router, _, _, up, down = self.names
+        return [
+            ParamSpec(self.name + ".router", (self.num_experts, h), "matrix_f32",
+                      (Source(self.prefix + router, self.num_experts),)),
+            ParamSpec(self.name + ".up", (self.inner, h), "matrix", self._sources(up, self.expert_size, self.shared_size)),
+            ParamSpec(self.name + ".down", (h, self.inner), "matrix",
+                      self._sources(down, self.expert_size, self.shared_size), axis=1),
+        ]
+
+    def bind(self, params, runtime) -> None:
+        self.router.bind(params[self.name + ".router"])
+        self.up.bind(params[self.name + ".up"])
+        self.down.bind(params[self.name + ".down"])
+
+    def forward(self, x, ctx):
+        weights = self.router(x, out_dtype=torch.float32)  # logits, float32 product
+        ops.route(weights, self.top, self.route_scale)
+        hidden = self.up(x)
+        ops.unary_act(hidden, hidden, self.activation, weights, self.expert_size)
+        return self.down.deferred(hidden, ctx)
+
+
+FEED_FORWARDS.register("two_layer", TwoLayer)
+FEED_FORWARDS.register("routed_experts", RoutedExperts)
 FEED_FORWARDS.register("swiglu", SwiGLU)
 FEED_FORWARDS.register("gated", SwiGLU)  # the same part under the name that fits either activation

@@ -12,7 +12,7 @@ import torch
 
 from ..kernels import ops
 from .base import NORMS, Norm, ParamSpec, Source
-from .lazy import DeferredProduct
+from .lazy import DeferredProduct, NormedDelta
 
 
 class RMSNorm(Norm):
@@ -42,6 +42,15 @@ class RMSNorm(Norm):
         self.dtype = runtime.dtype
 
     def forward(self, residual, delta, ctx, rows=None, scaled_ok=False):
+        if isinstance(delta, NormedDelta):
+            # the sub-layer's own norm, the add and this norm in one kernel
+            n = residual.shape[0] if rows is None else rows.numel()
+            out = torch.empty((n, self.size), dtype=self.dtype, device=residual.device)
+            y = delta.y
+            if y.dtype != self.dtype:
+                y = y.to(self.dtype)
+            ops.normed_add_rmsnorm(residual, y, delta.weight, delta.eps, self.weight, out, self.eps, rows)
+            return out
         if isinstance(delta, DeferredProduct):
             if (
                 scaled_ok and rows is None and delta.linear.out_features == self.size

@@ -116,9 +116,9 @@ def load_params(
                 other.append(f"checkpoint tensor {src.name!r} is claimed by two parameters")
             by_source[src.name] = (spec, offset, src.rows)
             offset += src.rows
-        if spec.sources and offset != spec.shape[0]:
+        if spec.sources and offset != spec.shape[spec.axis]:
             other.append(
-                f"parameter {spec.name!r}: its sources cover {offset} rows of {spec.shape[0]}"
+                f"parameter {spec.name!r}: its sources cover {offset} rows of {spec.shape[spec.axis]}"
             )
 
     out: dict[str, torch.Tensor] = {}
@@ -136,7 +136,7 @@ def load_params(
             continue
         seen.add(name)
         spec, offset, rows = hit
-        want = (rows, *spec.shape[1:])
+        want = spec.source_shape(rows)
         if tuple(tensor.shape) != want:
             wrong.append(
                 f"{name}: checkpoint has {tuple(tensor.shape)}, parameter {spec.name!r} "
@@ -161,7 +161,7 @@ def load_params(
             if dtype == torch.float32:
                 dest = dest.to(torch.float32)
                 out[spec.name] = dest
-        dest[offset : offset + rows].copy_(tensor, non_blocking=False)
+        dest.narrow(spec.axis, offset, rows).copy_(tensor, non_blocking=False)
 
     missing: list[str] = []
     for spec in specs:

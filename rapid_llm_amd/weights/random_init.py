@@ -54,8 +54,7 @@ def random_checkpoint_tensors(
         for src in spec.sources:
             if not src.name:
                 continue  # rows of zeros: the checkpoint ships nothing for them
-            shape = (src.rows, *spec.shape[1:])
-            t = _draw(shape, spec.init, gen, std, norm_std)
+            t = _draw(spec.source_shape(src.rows), spec.init, gen, std, norm_std)
             out[src.name] = t.to(_STORE[dtype]) if spec.role != "table" else t.to(torch.int32)
     return out
 
@@ -127,6 +126,6 @@ def random_params(
         offset = 0
         for src in spec.sources:
             if not src.name:  # rows no checkpoint tensor would feed are zeros here too
-                out[spec.name][offset : offset + src.rows] = 0
+                out[spec.name].narrow(spec.axis, offset, src.rows).zero_()
             offset += src.rows
     return out
