@@ -54,7 +54,7 @@ HEADERS = ("common.h", "static_entry.h")
 DEFAULT_HEAD_DIMS = tuple(range(16, 257, 16))
 
 # pairs of (key, value) head sizes of the tile attention that build_all() builds ahead of time
-DEFAULT_TILE_HEAD_DIMS = ((16, 32), (32, 16), (64, 32), (64, 64), (128, 64), (128, 128))
+DEFAULT_TILE_HEAD_DIMS = ((16, 16), (16, 48), (32, 16), (32, 32), (64, 32), (64, 64), (64, 128), (128, 64), (128, 128))
 
 _HIPCC_FLAGS = (
     "-O3",
