@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bfloat16]
                     [--shape NAME] [--batch B] [--prompt-len T] [--context C]
     python bench.py --workload qwen3-0.6b-256 | qwen3-32b-32
-    python bench.py --design fokulorn [--design-size 2b,8b]
+    python bench.py --design fokulorn|sikevik [--design-size 2b,8b]
 
 A "step" is one decode step of the whole batch through the engine's step function and the
 greedy sampling kernel, tokens fed back.  The default run has the layer sizes of
@@ -29,6 +29,12 @@ sizes of real models, beside the Qwen3 decoder of the same width, depth, heads a
 feed-forward width: prefill of one prompt and decode at batch 8 through the same step
 function, and the design's own kernels alone against their rooflines.  It prints one line of
 its own and leaves the default run as it is.
+
+``--design sikevik`` does the same for the Sikevik decoder (windowed attention that keeps a
+request's first positions, with a sink term and value heads of half the key heads' size; norms
+before and behind every sub-layer; one dense two-layer feed-forward, then mixtures of eight
+experts with a shared one; the last six layers in two passes of three), whose feed-forward
+matrices hold as many weights a layer as Qwen3's.
 
 Metric definitions follow rapid_llm's docs/benchmark_models.md:141-149: decode tok/s is
 batch / mean step time; prefill tok/s is prompt tokens / prefill latency; both timed
@@ -310,6 +316,76 @@ def fokulorn_body(z: dict) -> dict:
             "norm": {"eps": 1e-6}, "layers": layers}
 
 
+def sikevik_body(z: dict) -> dict:
+    """Eight layer runs as five layers, the last three twice; a layer's feed-forward matrices
+    hold what Qwen3's three do (two matrices of 1.5 x the width for the dense one; eight experts
+    of an eighth and a shared one of half the width for the others)."""
+    ff = z["ff"]
+    mixer = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["head_dim"], "vdim": z["head_dim"] // 2,
+             "scale": z["head_dim"] ** -0.5, "mask": {"size": z["window"], "keep_first": 64}}
+    moe = {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 8, "top": 2, "scale": 1.0},
+           "shared": {"ff": ff // 2}}
+    n = z["layers"] - 3
+    layers = [{"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff * 3 // 2} if i == 0 else moe}
+              for i in range(n)]
+    return {"architecture": "Sikevik", "width": z["width"], "vocab": z["vocab"], "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-6}, "layers": layers, "loop": {"start": n - 3, "stop": n, "times": 2}}
+
+
+def _time_sikevik_kernels(z: dict, prompt_len: int, batch: int) -> dict:
+    """The design's attention kernel alone: one prompt from its start (matrix rate over the keys
+    every query sees) and ``batch`` single tokens behind ``prompt_len`` (bytes of the keys and
+    values read), microseconds and share of the roofline."""
+    import types
+
+    import torch
+
+    from rapid_llm_amd.kernels import ops
+
+    nq, nkv, d, dv, page = z["heads"], z["kv_heads"], z["head_dim"], z["head_dim"] // 2, 16
+    window, keep, dev = z["window"], 64, "cuda"
+
+    def run(seqs):
+        tokens = sum(n for _, n in seqs)
+        per = -(-max(a + n for a, n in seqs) // page)
+        pages = len(seqs) * per + 1
+        table = (1 + torch.arange(len(seqs) * per, dtype=torch.int32, device=dev)).view(len(seqs), per).contiguous()
+        kc = (torch.randn(pages, nkv, page, d, device=dev) * 0.5).bfloat16()
+        vc = (torch.randn(pages, nkv, dv, page, device=dev) * 0.5).bfloat16()
+        q = (torch.randn(tokens, nq * d, device=dev) * 0.5).bfloat16()
+        out = torch.empty((tokens, nq * dv), dtype=torch.bfloat16, device=dev)
+        pos = torch.cat([torch.arange(a, a + n, dtype=torch.int32) for a, n in seqs]).to(dev)
+        slot = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, (_, n) in enumerate(seqs)]).to(dev)
+        ctx = types.SimpleNamespace(positions=pos, token_slot=slot, token_ids=pos, h_seq_starts=[a for a, _ in seqs],
+                                    h_seq_lens=[n for _, n in seqs], max_position=int(pos.max()), extra={})
+
+        def call():
+            ops.paged_attention(q, kc, vc, out, ctx, table, page, nq, nkv, d, window, d ** -0.5,
+                                value_dim=dv, keep_first=keep, sink=True)
+
+        for _ in range(3):
+            call()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(10):
+            call()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / 10
+
+    sec_p = run([(0, prompt_len)])
+    seen = sum(min(p + 1, window) + (min(keep, p + 1 - window) if p + 1 > window else 0) for p in range(prompt_len))
+    flops = 2.0 * nq * seen * (d + dv)
+    sec_d = run([(prompt_len, 1)] * batch)
+    keys = min(prompt_len + 1, window) + (keep if prompt_len + 1 > window + keep else 0)
+    kv_bytes = 2.0 * batch * nkv * keys * (d + dv)
+    return {
+        "attention_prefill_us": round(sec_p * 1e6, 1),
+        "attention_prefill_frac_bf16_matrix": round(flops / sec_p / (PEAK_TFLOPS["bfloat16"] * 1e12), 4),
+        "attention_decode_us": round(sec_d * 1e6, 1),
+        "attention_decode_frac_hbm": round(kv_bytes / sec_d / 1e9 / HBM_GBPS, 4),
+    }
+
+
 def qwen3_body(z: dict) -> dict:
     return dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=z["layers"],
                 hidden_size=z["width"], num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"],
@@ -430,22 +506,29 @@ def _time_kernels(z: dict, prompt_len: int, batch: int) -> dict:
     }
 
 
+DESIGNS = {
+    "fokulorn": ("Fokulorn", fokulorn_body, _time_kernels),
+    "sikevik": ("Sikevik", sikevik_body, _time_sikevik_kernels),
+}
+
+
 def run_design(args) -> int:
-    if args.design != "fokulorn":
-        print(f"unknown design {args.design!r}; known: fokulorn")
+    if args.design not in DESIGNS:
+        print(f"unknown design {args.design!r}; known: {', '.join(sorted(DESIGNS))}")
         return 2
+    title, design_body, design_kernels = DESIGNS[args.design]
     prompt_len = args.prompt_len or 2048
-    out = {"design": "Fokulorn", "beside": "Qwen3 of equal width, depth, heads and feed-forward width",
+    out = {"design": title, "beside": "Qwen3 of equal width, depth, heads and feed-forward width",
            "dtype": "bf16", "data": "synthetic (uniform random token ids, random N(0,0.02) weights)",
            "prompt_len": prompt_len, "batch": args.batch, "sizes": {}}
     for name in [x for x in args.design_size.split(",") if x]:
         z = DESIGN_SIZES[name]
         row = {"config": z}
-        row["fokulorn"] = _time_model(fokulorn_body(z), prompt_len, args.batch, args.point_steps, prompt_len + 512)
-        print(f"[bench] {name} fokulorn {row['fokulorn']}", file=sys.stderr, flush=True)
+        row[args.design] = _time_model(design_body(z), prompt_len, args.batch, args.point_steps, prompt_len + 512)
+        print(f"[bench] {name} {args.design} {row[args.design]}", file=sys.stderr, flush=True)
         row["qwen3"] = _time_model(qwen3_body(z), prompt_len, args.batch, args.point_steps, prompt_len + 512)
         print(f"[bench] {name} qwen3 {row['qwen3']}", file=sys.stderr, flush=True)
-        row["kernels"] = _time_kernels(z, prompt_len, args.batch)
+        row["kernels"] = design_kernels(z, prompt_len, args.batch)
         print(f"[bench] {name} kernels {row['kernels']}", file=sys.stderr, flush=True)
         out["sizes"][name] = row
     print(json.dumps(out), flush=True)
@@ -477,7 +560,7 @@ def main() -> int:
     ap.add_argument("--peaks", action="store_true",
                     help="measure what the device reaches with library kernels (a large read, copy and square products) and exit")
     ap.add_argument("--design", default=None,
-                    help="measure another architecture of the engine beside Qwen3 at equal size (fokulorn) and exit")
+                    help="measure another architecture of the engine beside Qwen3 at equal size (fokulorn, sikevik) and exit")
     ap.add_argument("--design-size", default="2b,8b", help=f"sizes for --design: {', '.join(DESIGN_SIZES)}")
     args = ap.parse_args()
     if args.peaks:

@@ -43,6 +43,10 @@ constexpr int D = RL_HEAD_DIM;
 constexpr int DV = RL_VALUE_DIM;
 constexpr int DB = D / 16;   // 16-channel chunks of the first product
 constexpr int VB = DV / 16;  // 16-channel blocks of the output
+// blocks of 16 rows a wave multiplies with every key tile it reads, in a bfloat16 step of
+// portions: as many as the registers hold beside two tiles of operands
+constexpr int PORTION_BLOCKS = (D + DV <= 192) ? 4 : ((D + DV <= 384) ? 2 : 1);
+constexpr int MAX_STAGED_PAGES = 2048;  // page ids of a tile's keys that are staged in LDS
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
@@ -99,7 +103,10 @@ __device__ inline float row_sum(float v) {
 
 // tile_info: [tiles][3] = index of the request's first token in the step, its tokens in the
 // step, first row of the tile.  The request's first position is read from `positions`.
-template <typename T, int AW>
+// A workgroup's tile is R blocks of 16 rows: every wave multiplies a key tile it has read with
+// all R blocks in turn, so that what is read from the cache serves R times the rows (a step of
+// portions is bound by those reads).  A row's sums do not depend on R.
+template <typename T, int AW, int R>
 __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     T* __restrict__ out, const int* __restrict__ tile_info, const int* __restrict__ positions,
@@ -110,8 +117,8 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
     const int hk = blockIdx.y;
     const int G = nq / nkv;
     const int at = tile_info[3 * tile], n = tile_info[3 * tile + 1], row0 = tile_info[3 * tile + 2];
-    __shared__ float fold_ml[AW - 1][2][RL_WAVE];
-    __shared__ float fold_acc[AW - 1][VB * 4][RL_WAVE];
+    __shared__ float fold_ml[AW - 1][R][2][RL_WAVE];
+    __shared__ float fold_acc[AW - 1][R][VB * 4][RL_WAVE];
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
     const int r16 = lane & 15;
@@ -120,42 +127,72 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
     const int* table = block_table + (size_t)token_slot[at] * table_stride;
 
     const int rows = n * G;
-    const int row = row0 + r16;
-    const bool row_ok = row < rows;
-    const int tok = (row_ok ? row : rows - 1) / G;
-    const int head = hk * G + (row_ok ? row : rows - 1) % G;
-    const int pos = start + tok;
-    const int kend = pos + 1;
-    const int kstart = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
     const int keep = window > 0 ? keep_first : 0;  // keys below it are seen from anywhere
+    bool row_ok[R];
+    int tok[R], head[R], kend[R], kstart[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int row = row0 + 16 * r + r16;
+        row_ok[r] = row < rows;
+        tok[r] = (row_ok[r] ? row : rows - 1) / G;
+        head[r] = hk * G + (row_ok[r] ? row : rows - 1) % G;
+        const int pos = start + tok[r];
+        kend[r] = pos + 1;
+        kstart[r] = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    }
+    const int blocks = min(R, (rows - row0 + 15) / 16);  // blocks of the tile that hold rows
 
     // the keys any row of the tile sees: the kept first ones, and from the first row's first key
     // (rows ascend with the tokens), in whole tiles of 16, up to the last row's own position
     const int first_pos = start + row0 / G;
-    const int last_pos = start + (min(rows, row0 + 16) - 1) / G;
+    const int last_pos = start + (min(rows, row0 + 16 * R) - 1) / G;
     const int first_key = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
     const int lo = first_key & ~15;
     const int hi = last_pos + 1;                     // keys below hi are in the cache
     const int kept_end = min((keep + 15) & ~15, lo);  // tiles [0, kept_end) come before those of [lo, hi)
 
-    // Q^T: lane (row r16, g) holds channels 16c + 4g .. + 3 of its row
-    quad qf[DB];
-    {
-        const T* qrow = q + ((size_t)(at + tok) * nq + head) * D + 4 * g;
+    // The page ids of both runs of keys, staged once: a step then waits for its keys and values
+    // alone, not for a table entry first.  A tile with more pages than fit reads the table itself.
+    __shared__ int s_pages[MAX_STAGED_PAGES];
+    const int kept_pages = (kept_end + page_size - 1) / page_size;
+    const int lo_page = lo / page_size;
+    const int late_pages = (hi + page_size - 1) / page_size - lo_page;
+    const bool staged = kept_pages + late_pages <= MAX_STAGED_PAGES;
+    if (staged) {
+        for (int i = threadIdx.x; i < kept_pages + late_pages; i += AW * RL_WAVE)
+            s_pages[i] = table[i < kept_pages ? i : lo_page + (i - kept_pages)];
+        __syncthreads();
+    }
+    auto page_of = [&](int key) -> int {
+        const int idx = key / page_size;
+        if (!staged) return table[idx];
+        return s_pages[idx >= lo_page ? kept_pages + (idx - lo_page) : idx];
+    };
+
+    // Q^T: lane (row r16, g) holds channels 16c + 4g .. + 3 of its row of every block
+    quad qf[R][DB];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const T* qrow = q + ((size_t)(at + tok[r]) * nq + head[r]) * D + 4 * g;
 #pragma unroll
         for (int c = 0; c < DB; ++c) {
-            qf[c] = ld_quad<T>(qrow + 16 * c);
-            if (!row_ok) {
+            qf[r][c] = ld_quad<T>(qrow + 16 * c);
+            if (!row_ok[r]) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) qf[c][i] = 0;
+                for (int i = 0; i < 4; ++i) qf[r][c][i] = 0;
             }
         }
     }
 
-    float m = -INFINITY, l = 0.f;
-    f32x4 acc[VB];
+    float m[R], l[R];
+    f32x4 acc[R][VB];
 #pragma unroll
-    for (int b = 0; b < VB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < R; ++r) {
+        m[r] = -INFINITY;
+        l[r] = 0.f;
+#pragma unroll
+        for (int b = 0; b < VB; ++b) acc[r][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
 
     // operands of one tile of 16 keys: lane (key r16, g) reads channels 16c + 4g .. + 3 of its
     // key; lane (channel r16, g) reads keys kb + 4g .. + 3 of its channel in every block
@@ -165,65 +202,69 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
     auto load = [&](int kb, Frags& f) {
         const int key = min(kb + r16, hi - 1);  // beyond the cache: any real key, masked below
         const T* krow =
-            k_cache + (((size_t)table[key / page_size] * nkv + hk) * page_size + key % page_size) * D + 4 * g;
+            k_cache + (((size_t)page_of(key) * nkv + hk) * page_size + key % page_size) * D + 4 * g;
 #pragma unroll
         for (int c = 0; c < DB; ++c) f.k[c] = ld_quad<T>(krow + 16 * c);
         const int key4 = min(kb + 4 * g, (hi - 1) & ~3);
-        const T* vrow = v_cache + (((size_t)table[key4 / page_size] * nkv + hk) * DV + r16) * page_size +
+        const T* vrow = v_cache + (((size_t)page_of(key4) * nkv + hk) * DV + r16) * page_size +
                         key4 % page_size;
 #pragma unroll
         for (int b = 0; b < VB; ++b) f.v[b] = ld_quad<T>(vrow + (size_t)16 * b * page_size);
     };
 
-    // S^T = K Q^T of one tile, the chunks dealt to four accumulators that are added at the
-    // end (one chain of dependent instructions would leave the matrix core idle)
-    auto scores = [&](const Frags& f) -> f32x4 {
+    // S^T = K Q^T of one tile and one block of rows, the chunks dealt to four accumulators that
+    // are added at the end (one chain of dependent instructions would leave the matrix core idle)
+    auto scores = [&](const Frags& f, int r) -> f32x4 {
         f32x4 part[4];
 #pragma unroll
         for (int a4 = 0; a4 < 4; ++a4) part[a4] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int c = 0; c < DB; ++c) part[c & 3] = mma(f.k[c], qf[c], part[c & 3]);
+        for (int c = 0; c < DB; ++c) part[c & 3] = mma(f.k[c], qf[r][c], part[c & 3]);
         return (part[0] + part[1]) + (part[2] + part[3]);
     };
 
-    // softmax and second product of the tile at kb, given its scores and its values
-    auto finish_tile = [&](int kb, f32x4 s, const quad (&vcur)[VB]) {
+    // softmax and second product of the tile at kb for block r, given its scores and its values
+    auto finish_block = [&](int kb, int r, f32x4 s, const quad (&vcur)[VB]) {
         // ---- this lane's keys kb + 4g + i of its own row ------------------------------------
         float tmax = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int key = kb + 4 * g + i;
-            const bool seen = row_ok && key < kend && (key >= kstart || key < keep);
+            const bool seen = row_ok[r] && key < kend[r] && (key >= kstart[r] || key < keep);
             s[i] = seen ? s[i] * scale : -INFINITY;
             tmax = fmaxf(tmax, s[i]);
         }
         tmax = row_max(tmax);
-        const float m_new = fmaxf(m, tmax);
+        const float m_new = fmaxf(m[r], tmax);
         float alpha = 1.f;  // no visible key so far and none here: nothing changes
         f32x4 p = (f32x4){0.f, 0.f, 0.f, 0.f};
         if (m_new != -INFINITY) {
-            alpha = expf(m - m_new);  // m = -inf before the row's first key: 0
+            alpha = expf(m[r] - m_new);  // m = -inf before the row's first key: 0
 #pragma unroll
             for (int i = 0; i < 4; ++i) p[i] = expf(s[i] - m_new);  // masked: exactly 0
         }
-        l = l * alpha + row_sum((p[0] + p[1]) + (p[2] + p[3]));
-        m = m_new;
+        l[r] = l[r] * alpha + row_sum((p[0] + p[1]) + (p[2] + p[3]));
+        m[r] = m_new;
         quad pq;
         to_quad(p, pq);
         // ---- O^T = O^T alpha + V^T P^T --------------------------------------------------------
 #pragma unroll
         for (int b = 0; b < VB; ++b) {
-            quad vf = vcur[b];
-            // keys no row of the tile sees (beyond the cache, or between the kept ones and the
-            // window, whose pages may have been given back) may hold anything: 0 * it must be 0
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = kb + 4 * g + i;
-                if (key >= hi || (key < first_key && key >= keep)) vf[i] = 0;
+            for (int i = 0; i < 4; ++i) acc[r][b][i] *= alpha;
+            acc[r][b] = mma(vcur[b], pq, acc[r][b]);
+        }
+    };
+    // keys no row of the tile sees (beyond the cache, or between the kept ones and the window,
+    // whose pages may have been given back) may hold anything: 0 * it must be 0
+    auto clean = [&](int kb, quad (&v)[VB]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int key = kb + 4 * g + i;
+            if (key >= hi || (key < first_key && key >= keep)) {
+#pragma unroll
+                for (int b = 0; b < VB; ++b) v[b][i] = 0;
             }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[b][i] *= alpha;
-            acc[b] = mma(vf, pq, acc[b]);
         }
     };
 
@@ -238,75 +279,106 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
     auto kb_of = [&](int i) -> int {
         return i < kept_tiles ? kept_mine + i * STEP : mine + (i - kept_tiles) * STEP;
     };
-    // Software pipeline over the wave's tiles: while a tile goes through softmax and the second
-    // product, the scores of the next have been multiplied and the operands of the one after
-    // are in flight.  The last two tiles stand outside the loop, so that inside it the loads
-    // are issued without a condition.
-    if (total > 0) {
-        int left = total;  // tiles of this wave, the current one included
-        int i = 0;
-        Frags nxt;
-        quad vcur[VB], vnext[VB];
-        load(kb_of(0), nxt);
-        f32x4 sc = scores(nxt);
+    if constexpr (R == 1) {
+        // Software pipeline over the wave's tiles: while a tile goes through softmax and the
+        // second product, the scores of the next have been multiplied and the operands of the one
+        // after are in flight.  The last two tiles stand outside the loop, so that inside it the
+        // loads are issued without a condition.
+        if (total > 0) {
+            int left = total;  // tiles of this wave, the current one included
+            int i = 0;
+            Frags nxt;
+            quad vcur[VB], vnext[VB];
+            load(kb_of(0), nxt);
+            f32x4 sc = scores(nxt, 0);
 #pragma unroll
-        for (int b = 0; b < VB; ++b) vcur[b] = nxt.v[b];
-        if (left > 1) load(kb_of(1), nxt);
-        while (left > 2) {
-            const f32x4 s_next = scores(nxt);
+            for (int b = 0; b < VB; ++b) vcur[b] = nxt.v[b];
+            if (left > 1) load(kb_of(1), nxt);
+            while (left > 2) {
+                const f32x4 s_next = scores(nxt, 0);
 #pragma unroll
-            for (int b = 0; b < VB; ++b) vnext[b] = nxt.v[b];
-            load(kb_of(i + 2), nxt);
-            __builtin_amdgcn_sched_barrier(0);
-            finish_tile(kb_of(i), sc, vcur);
-            sc = s_next;
+                for (int b = 0; b < VB; ++b) vnext[b] = nxt.v[b];
+                load(kb_of(i + 2), nxt);
+                __builtin_amdgcn_sched_barrier(0);
+                clean(kb_of(i), vcur);
+                finish_block(kb_of(i), 0, sc, vcur);
+                sc = s_next;
 #pragma unroll
-            for (int b = 0; b < VB; ++b) vcur[b] = vnext[b];
-            ++i;
-            --left;
+                for (int b = 0; b < VB; ++b) vcur[b] = vnext[b];
+                ++i;
+                --left;
+            }
+            if (left == 2) {
+                const f32x4 s_next = scores(nxt, 0);
+                clean(kb_of(i), vcur);
+                finish_block(kb_of(i), 0, sc, vcur);
+                clean(kb_of(i + 1), nxt.v);
+                finish_block(kb_of(i + 1), 0, s_next, nxt.v);
+            } else {
+                clean(kb_of(i), vcur);
+                finish_block(kb_of(i), 0, sc, vcur);
+            }
         }
-        if (left == 2) {
-            const f32x4 s_next = scores(nxt);
-            finish_tile(kb_of(i), sc, vcur);
-            finish_tile(kb_of(i + 1), s_next, nxt.v);
-        } else {
-            finish_tile(kb_of(i), sc, vcur);
+    } else {
+        // several blocks of rows: the next tile's operands travel while this one is multiplied
+        // with every block in turn
+        if (total > 0) {
+            Frags cur, nxt;
+            load(kb_of(0), cur);
+            for (int i = 0; i < total; ++i) {
+                const int kb = kb_of(i);
+                load(kb_of(min(i + 1, total - 1)), nxt);  // the last one again: no load behind a condition
+                __builtin_amdgcn_sched_barrier(0);
+                clean(kb, cur.v);
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    if (r < blocks) finish_block(kb, r, scores(cur, r), cur.v);
+                cur = nxt;
+            }
         }
     }
     // ---- fold the waves' states in their order (a wave without visible keys has m = -inf,
     // l = 0 and zero sums: it changes nothing, exactly) ----------------------------------------
     if (wave > 0) {
-        fold_ml[wave - 1][0][lane] = m;
-        fold_ml[wave - 1][1][lane] = l;
 #pragma unroll
-        for (int b = 0; b < VB; ++b)
+        for (int r = 0; r < R; ++r) {
+            fold_ml[wave - 1][r][0][lane] = m[r];
+            fold_ml[wave - 1][r][1][lane] = l[r];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fold_acc[wave - 1][4 * b + i][lane] = acc[b][i];
+            for (int b = 0; b < VB; ++b)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) fold_acc[wave - 1][r][4 * b + i][lane] = acc[r][b][i];
+        }
     }
     __syncthreads();
     if (wave > 0) return;
 #pragma unroll
-    for (int w = 0; w < AW - 1; ++w) {
-        const float m_w = fold_ml[w][0][lane], l_w = fold_ml[w][1][lane];
-        const float m_new = fmaxf(m, m_w);
-        if (m_new == -INFINITY) continue;
-        const float fa = expf(m - m_new), fb = expf(m_w - m_new);
-        l = l * fa + l_w * fb;
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int w = 0; w < AW - 1; ++w) {
+            const float m_w = fold_ml[w][r][0][lane], l_w = fold_ml[w][r][1][lane];
+            const float m_new = fmaxf(m[r], m_w);
+            if (m_new == -INFINITY) continue;
+            const float fa = expf(m[r] - m_new), fb = expf(m_w - m_new);
+            l[r] = l[r] * fa + l_w * fb;
+#pragma unroll
+            for (int b = 0; b < VB; ++b)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[r][b][i] = acc[r][b][i] * fa + fold_acc[w][r][4 * b + i][lane] * fb;
+            m[r] = m_new;
+        }
+        if (!row_ok[r]) continue;
+        // the key of score 0 that has no value: exp(0 - m) more in the denominator
+        if (sink) l[r] += expf(-m[r]);
+        // acc[r][b][i] is channel 16b + 4g + i of the lane's row
+        T* orow = out + ((size_t)(at + tok[r]) * nq + head[r]) * DV + 4 * g;
+        const float inv = 1.f / l[r];
 #pragma unroll
         for (int b = 0; b < VB; ++b)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[b][i] = acc[b][i] * fa + fold_acc[w][4 * b + i][lane] * fb;
-        m = m_new;
+            store_quad(orow + 16 * b, (f32x4){acc[r][b][0] * inv, acc[r][b][1] * inv, acc[r][b][2] * inv,
+                                              acc[r][b][3] * inv});
     }
-    if (!row_ok) return;
-    // the key of score 0 that has no value: exp(0 - m) more in the denominator
-    if (sink) l += expf(-m);
-    // acc[b][i] is channel 16b + 4g + i of the lane's row
-    T* orow = out + ((size_t)(at + tok) * nq + head) * DV + 4 * g;
-    const float inv = 1.f / l;
-#pragma unroll
-    for (int b = 0; b < VB; ++b)
-        store_quad(orow + 16 * b, (f32x4){acc[b][0] * inv, acc[b][1] * inv, acc[b][2] * inv, acc[b][3] * inv});
 }
 
 }  // namespace tileattn
@@ -316,27 +388,46 @@ extern "C" int rl_attn_tile_value_dim() { return tileattn::DV; }
 
 // Every token of the step, single tokens and portions alike.  page_size must be a multiple
 // of 4 (the four keys of a lane lie in one page).
+// rows of a workgroup's tile in a bfloat16 launch of portions (tile_rows > 16)
+extern "C" int rl_attn_tile_wide_rows() { return 16 * tileattn::PORTION_BLOCKS; }
+
+// Every token of the step, single tokens and portions alike.  page_size must be a multiple
+// of 4 (the four keys of a lane lie in one page).  tile_rows: the rows of a tile of tile_info,
+// 16 or, in bfloat16, rl_attn_tile_wide_rows().
 extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_cache, void* out,
                             const int* tile_info, int num_tiles, const int* positions,
                             const int* token_slot, const int* block_table, int table_stride,
                             int page_size, int nq, int nkv, int window, int keep_first, int sink,
-                            float scale, int act_type, hipStream_t stream) {
+                            float scale, int wide, int tile_rows, int act_type, hipStream_t stream) {
     if (num_tiles <= 0) return RL_OK;
     if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535 || window < 0 || keep_first < 0)
         return RL_ERR_ARG;
     constexpr int AW = 4;
+    constexpr int PB = tileattn::PORTION_BLOCKS;
     dim3 grid(num_tiles, nkv), block(AW * RL_WAVE);
+#define RL_TILE_ARGS(TYPE)                                                                                  \
+    (const TYPE*)q, (const TYPE*)k_cache, (const TYPE*)v_cache, (TYPE*)out, tile_info, positions, token_slot, \
+        block_table, table_stride, page_size, nq, nkv, window, keep_first, sink, scale
+    if (act_type == RL_BF16 && tile_rows == 16 * PB && PB > 1) {
+        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, PB>), grid, block, 0, stream, RL_TILE_ARGS(bf16_t));
+        return rl_launch_status();
+    }
+    if (tile_rows != 16) return RL_ERR_ARG;
+    // `wide` (bfloat16 only: the order of the sums changes with the number of waves): a launch of
+    // few tiles over many keys (single tokens) deals every tile's keys to as many waves as the
+    // fold's buffers allow, so that a wave walks a quarter of the steps
+    if (wide && act_type == RL_BF16) {
+        constexpr int WIDE = tileattn::DV <= 128 ? 16 : 8;
+        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, WIDE, 1>), grid, dim3(WIDE * RL_WAVE), 0, stream,
+                           RL_TILE_ARGS(bf16_t));
+        return rl_launch_status();
+    }
     if (act_type == RL_F32)
-        hipLaunchKernelGGL((tileattn::attn_tile_kernel<float, AW>), grid, block, 0, stream, (const float*)q,
-                           (const float*)k_cache, (const float*)v_cache, (float*)out, tile_info, positions,
-                           token_slot, block_table, table_stride, page_size, nq, nkv, window, keep_first, sink,
-                           scale);
+        hipLaunchKernelGGL((tileattn::attn_tile_kernel<float, AW, 1>), grid, block, 0, stream, RL_TILE_ARGS(float));
     else if (act_type == RL_BF16)
-        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW>), grid, block, 0, stream, (const bf16_t*)q,
-                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_info, positions,
-                           token_slot, block_table, table_stride, page_size, nq, nkv, window, keep_first, sink,
-                           scale);
+        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, 1>), grid, block, 0, stream, RL_TILE_ARGS(bf16_t));
     else
         return RL_ERR_ARG;
+#undef RL_TILE_ARGS
     return rl_launch_status();
 }

@@ -271,19 +271,103 @@ __global__ void normed_add_rmsnorm_kernel(float* __restrict__ residual, const T*
         o[i] = from_float<T>(res[i] * rrms * weight[i]);
 }
 
+// The same with four elements a thread and load, a row of up to 16 * blockDim elements held in
+// registers from its first read to its last use.
+template <typename T, int CHUNKS>
+__global__ void normed_add_rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ y,
+                                              const float* __restrict__ w_y, float eps_y,
+                                              const float* __restrict__ weight, T* __restrict__ out,
+                                              const int* __restrict__ rows, int hidden, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int row = rows ? rows[r] : r;
+    float4* res = reinterpret_cast<float4*>(residual + (size_t)row * hidden);
+    const Vec4<T>* yr = reinterpret_cast<const Vec4<T>*>(y + (size_t)row * hidden);
+    const float4* wy4 = reinterpret_cast<const float4*>(w_y);
+    const float4* w4 = reinterpret_cast<const float4*>(weight);
+    const int nvec = hidden >> 2;
+    float4 val[CHUNKS], old[CHUNKS], wy[CHUNKS], wt[CHUNKS];
+    float ss = 0.f;
+    // everything the row needs is asked for before the first sum's barrier
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nvec) {
+            const Vec4<T> v = yr[i];
+            val[c] = make_float4(to_float(v.v[0]), to_float(v.v[1]), to_float(v.v[2]), to_float(v.v[3]));
+            old[c] = res[i];
+            wy[c] = wy4[i];
+            if (out) wt[c] = w4[i];
+            ss += val[c].x * val[c].x + val[c].y * val[c].y + val[c].z * val[c].z + val[c].w * val[c].w;
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float rr_y = rsqrtf(ss / (float)hidden + eps_y);
+    float s2 = 0.f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nvec) {
+            float4 v;
+            v.x = old[c].x + val[c].x * rr_y * wy[c].x;
+            v.y = old[c].y + val[c].y * rr_y * wy[c].y;
+            v.z = old[c].z + val[c].z * rr_y * wy[c].z;
+            v.w = old[c].w + val[c].w * rr_y * wy[c].w;
+            res[i] = v;
+            val[c] = v;
+            s2 += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+    }
+    if (!out) return;
+    s2 = block_sum(s2, scratch);
+    const float rrms = rsqrtf(s2 / (float)hidden + eps);
+    Vec4<T>* o = reinterpret_cast<Vec4<T>*>(out + (size_t)r * hidden);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nvec) {
+            Vec4<T> v;
+            v.v[0] = from_float<T>(val[c].x * rrms * wt[c].x);
+            v.v[1] = from_float<T>(val[c].y * rrms * wt[c].y);
+            v.v[2] = from_float<T>(val[c].z * rrms * wt[c].z);
+            v.v[3] = from_float<T>(val[c].w * rrms * wt[c].w);
+            o[i] = v;
+        }
+    }
+}
+
+template <typename T>
+static void launch_normed_add_rmsnorm(float* residual, const T* y, const float* w_y, float eps_y,
+                                      const float* weight, T* out, const int* rows, int out_rows, int hidden,
+                                      float eps, hipStream_t stream) {
+    dim3 grid(out_rows);
+    if (hidden % 4 == 0 && hidden <= 16 * 1024) {
+        const int nvec = hidden / 4;
+        const int threads = ((nvec + RL_WAVE - 1) / RL_WAVE) * RL_WAVE;
+        if (threads <= 1024)
+            hipLaunchKernelGGL((normed_add_rmsnorm_vec_kernel<T, 1>), grid, dim3(threads), 0, stream, residual, y,
+                               w_y, eps_y, weight, out, rows, hidden, eps);
+        else
+            hipLaunchKernelGGL((normed_add_rmsnorm_vec_kernel<T, 4>), grid, dim3(1024), 0, stream, residual, y,
+                               w_y, eps_y, weight, out, rows, hidden, eps);
+        return;
+    }
+    const int threads = hidden >= 4096 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 256 : 64));
+    hipLaunchKernelGGL((normed_add_rmsnorm_kernel<T, 8>), grid, dim3(threads), 0, stream, residual, y, w_y, eps_y,
+                       weight, out, rows, hidden, eps);
+}
+
 extern "C" int rl_normed_add_rmsnorm(float* residual, const void* y, const float* w_y, float eps_y,
                                      const float* weight, void* out, const int* rows, int out_rows,
                                      int hidden, float eps, int act_type, hipStream_t stream) {
     if (out_rows <= 0) return RL_OK;
     if (out && !weight) return RL_ERR_ARG;
-    dim3 grid(out_rows);
-    const int threads = hidden >= 4096 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 256 : 64));
     if (act_type == RL_F32)
-        hipLaunchKernelGGL((normed_add_rmsnorm_kernel<float, 8>), grid, dim3(threads), 0, stream, residual,
-                           (const float*)y, w_y, eps_y, weight, (float*)out, rows, hidden, eps);
+        launch_normed_add_rmsnorm<float>(residual, (const float*)y, w_y, eps_y, weight, (float*)out, rows, out_rows,
+                                         hidden, eps, stream);
     else if (act_type == RL_BF16)
-        hipLaunchKernelGGL((normed_add_rmsnorm_kernel<bf16_t, 8>), grid, dim3(threads), 0, stream, residual,
-                           (const bf16_t*)y, w_y, eps_y, weight, (bf16_t*)out, rows, hidden, eps);
+        launch_normed_add_rmsnorm<bf16_t>(residual, (const bf16_t*)y, w_y, eps_y, weight, (bf16_t*)out, rows,
+                                          out_rows, hidden, eps, stream);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -303,19 +387,44 @@ __global__ void pair_rows_kernel(const float* __restrict__ a, const float* __res
     }
 }
 
+// four channels a thread (hidden a multiple of 4); `total` counts groups of four
+template <typename T>
+__global__ void pair_rows_vec_kernel(const float4* __restrict__ a, const float4* __restrict__ b,
+                                     Vec4<T>* __restrict__ out, size_t total, int hidden4) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; idx < total; idx += step) {
+        const size_t t = idx / (2 * (size_t)hidden4);
+        const int c = (int)(idx - t * 2 * (size_t)hidden4);
+        const float4 v = c < hidden4 ? a[t * hidden4 + c] : b[t * hidden4 + c - hidden4];
+        Vec4<T> o;
+        o.v[0] = from_float<T>(v.x);
+        o.v[1] = from_float<T>(v.y);
+        o.v[2] = from_float<T>(v.z);
+        o.v[3] = from_float<T>(v.w);
+        out[idx] = o;
+    }
+}
+
 extern "C" int rl_pair_rows(const float* a, const float* b, void* out, int tokens, int hidden,
                             int act_type, hipStream_t stream) {
     if (tokens <= 0 || hidden <= 0) return RL_OK;
-    const size_t total = (size_t)tokens * 2 * hidden;
+    if (act_type != RL_F32 && act_type != RL_BF16) return RL_ERR_ARG;
+    const bool vec = hidden % 4 == 0;
+    const size_t total = (size_t)tokens * 2 * hidden / (vec ? 4 : 1);
     size_t blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     dim3 grid((unsigned)blocks), block(256);
-    if (act_type == RL_F32)
+    if (vec && act_type == RL_F32)
+        hipLaunchKernelGGL(pair_rows_vec_kernel<float>, grid, block, 0, stream, (const float4*)a, (const float4*)b,
+                           (Vec4<float>*)out, total, hidden / 4);
+    else if (vec)
+        hipLaunchKernelGGL(pair_rows_vec_kernel<bf16_t>, grid, block, 0, stream, (const float4*)a, (const float4*)b,
+                           (Vec4<bf16_t>*)out, total, hidden / 4);
+    else if (act_type == RL_F32)
         hipLaunchKernelGGL(pair_rows_kernel<float>, grid, block, 0, stream, a, b, (float*)out, total, hidden);
-    else if (act_type == RL_BF16)
-        hipLaunchKernelGGL(pair_rows_kernel<bf16_t>, grid, block, 0, stream, a, b, (bf16_t*)out, total, hidden);
     else
-        return RL_ERR_ARG;
+        hipLaunchKernelGGL(pair_rows_kernel<bf16_t>, grid, block, 0, stream, a, b, (bf16_t*)out, total, hidden);
     return rl_launch_status();
 }
 
@@ -510,23 +619,54 @@ __global__ void unary_act_kernel(const T* __restrict__ x, T* __restrict__ out, s
     }
 }
 
+// eight columns a thread: rows of a multiple of 8 columns, experts of a multiple of 8 hidden
+// units, so that a group of eight belongs to one expert; `total` counts groups
+template <typename T>
+__global__ void unary_act_vec_kernel(const T* __restrict__ x, T* __restrict__ out, size_t total, int cols8,
+                                     int kind, const float* __restrict__ route, int experts, int ff8) {
+    struct alignas(sizeof(T) * 8) Pack {
+        T v[8];
+    };
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; idx < total; idx += step) {
+        const Pack in = reinterpret_cast<const Pack*>(x)[idx];
+        float factor = 1.f;
+        if (route) {
+            const size_t t = idx / cols8;
+            const int c = (int)(idx - t * cols8);
+            if (c < experts * ff8) factor = route[t * experts + c / ff8];
+        }
+        Pack o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o.v[j] = from_float<T>(unary_act(to_float(in.v[j]), kind) * factor);
+        reinterpret_cast<Pack*>(out)[idx] = o;
+    }
+}
+
 extern "C" int rl_unary_act(const void* x, void* out, int tokens, int cols, int kind, const float* route,
                             int experts, int ff, int act_type, hipStream_t stream) {
     if (tokens <= 0 || cols <= 0) return RL_OK;
     if (kind < 0 || kind > 1) return RL_ERR_ARG;
     if (route && (experts < 1 || ff < 1 || (long)experts * ff > cols)) return RL_ERR_ARG;
-    const size_t total = (size_t)tokens * cols;
+    if (act_type != RL_F32 && act_type != RL_BF16) return RL_ERR_ARG;
+    const bool vec = cols % 8 == 0 && (!route || ff % 8 == 0);
+    const size_t total = (size_t)tokens * cols / (vec ? 8 : 1);
     size_t blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     dim3 grid((unsigned)blocks), block(256);
-    if (act_type == RL_F32)
+    if (vec && act_type == RL_F32)
+        hipLaunchKernelGGL(unary_act_vec_kernel<float>, grid, block, 0, stream, (const float*)x, (float*)out, total,
+                           cols / 8, kind, route, experts, ff / 8);
+    else if (vec)
+        hipLaunchKernelGGL(unary_act_vec_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)x, (bf16_t*)out,
+                           total, cols / 8, kind, route, experts, ff / 8);
+    else if (act_type == RL_F32)
         hipLaunchKernelGGL(unary_act_kernel<float>, grid, block, 0, stream, (const float*)x, (float*)out, total,
                            cols, kind, route, experts, ff);
-    else if (act_type == RL_BF16)
+    else
         hipLaunchKernelGGL(unary_act_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)x, (bf16_t*)out,
                            total, cols, kind, route, experts, ff);
-    else
-        return RL_ERR_ARG;
     return rl_launch_status();
 }
 
@@ -537,10 +677,8 @@ extern "C" int rl_unary_act(const void* x, void* out, int tokens, int cols, int 
 // z is overwritten by route.
 // --------------------------------------------------------------------------- //
 #define ROUTE_MAX_EXPERTS 1024
-__global__ void route_kernel(float* __restrict__ z, int tokens, int experts, int top, float scale) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= tokens) return;
-    float* row = z + (size_t)t * experts;
+// (a chosen expert's score is marked by its sign: scores are exponentials, never below +0)
+__device__ inline void route_row(float* __restrict__ row, float* __restrict__ dst, int experts, int top, float scale) {
     float m = -INFINITY;
     for (int e = 0; e < experts; ++e) m = fmaxf(m, row[e]);
     float total = 0.f;
@@ -549,31 +687,105 @@ __global__ void route_kernel(float* __restrict__ z, int tokens, int experts, int
         row[e] = p;
         total += p;
     }
-    unsigned chosen[ROUTE_MAX_EXPERTS / 32];
-    for (int w = 0; w < (experts + 31) / 32; ++w) chosen[w] = 0u;
     float sum = 0.f;
     for (int k = 0; k < top; ++k) {
-        int best = -1;
+        int best = 0;
         float best_s = -1.f;
         for (int e = 0; e < experts; ++e) {
-            if (chosen[e >> 5] >> (e & 31) & 1u) continue;
-            if (row[e] > best_s) {
-                best_s = row[e];
+            const float p = row[e];
+            if (!signbit(p) && p > best_s) {
+                best_s = p;
                 best = e;
             }
         }
-        chosen[best >> 5] |= 1u << (best & 31);
+        row[best] = -best_s;
         sum += best_s / total;
     }
     const float inv = scale / (sum + 1e-20f);
-    for (int e = 0; e < experts; ++e)
-        row[e] = (chosen[e >> 5] >> (e & 31) & 1u) ? row[e] / total * inv : 0.f;
+    for (int e = 0; e < experts; ++e) {
+        const float p = row[e];
+        dst[e] = signbit(p) ? -p / total * inv : 0.f;
+    }
+}
+
+__global__ void route_kernel(float* __restrict__ z, int tokens, int experts, int top, float scale) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= tokens) return;
+    route_row(z + (size_t)t * experts, z + (size_t)t * experts, experts, top, scale);
 }
 
 extern "C" int rl_route(float* z, int tokens, int experts, int top, float scale, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (experts < 1 || experts > ROUTE_MAX_EXPERTS || top < 1 || top > experts) return RL_ERR_ARG;
     hipLaunchKernelGGL(route_kernel, dim3((tokens + 63) / 64), dim3(64), 0, stream, z, tokens, experts, top, scale);
+    return rl_launch_status();
+}
+
+// The router's product and the weights in one kernel: a wave takes a token, computes
+// z_e = w[e] . x[t] in float32 for every expert (lanes stride the row, their sums are folded by
+// the wave: one order of summation per token whatever else is in the step), and its first
+// lane turns the logits into weights.  x may be bfloat16 or float32; w is float32.
+template <typename T>
+__global__ __launch_bounds__(256) void router_kernel(const T* __restrict__ x, const float* __restrict__ w,
+                                                     float* __restrict__ route, int tokens, int k, int experts,
+                                                     int top, float scale) {
+    extern __shared__ float s_logits[];  // [4][experts]
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    const int wave = threadIdx.x / RL_WAVE;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= tokens) return;  // whole waves leave; nothing below waits for another wave
+    float* z = s_logits + (size_t)wave * experts;
+    const T* xr = x + (size_t)t * k;
+    // eight experts at a time, so that a chunk of x is read once for eight rows of w and the
+    // loads of an iteration do not wait for each other
+    for (int e0 = 0; e0 < experts; e0 += 8) {
+        float acc[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+        const int ne = min(8, experts - e0);
+        if (k % 4 == 0) {
+            for (int i = 4 * lane; i < k; i += 4 * RL_WAVE) {
+                const Vec4<T> xv = *reinterpret_cast<const Vec4<T>*>(xr + i);
+                float4 wv[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    wv[j] = *reinterpret_cast<const float4*>(w + (size_t)(e0 + min(j, ne - 1)) * k + i);
+                const float x0 = to_float(xv.v[0]), x1 = to_float(xv.v[1]), x2 = to_float(xv.v[2]),
+                            x3 = to_float(xv.v[3]);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    acc[j] = fmaf(x3, wv[j].w, fmaf(x2, wv[j].z, fmaf(x1, wv[j].y, fmaf(x0, wv[j].x, acc[j]))));
+            }
+        } else {
+            for (int i = lane; i < k; i += RL_WAVE) {
+                const float xv = to_float(xr[i]);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[j] = fmaf(xv, w[(size_t)(e0 + min(j, ne - 1)) * k + i], acc[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float sum = wave_sum(acc[j]);
+            if (lane == 0 && j < ne) z[e0 + j] = sum;
+        }
+    }
+    if (lane == 0) route_row(z, route + (size_t)t * experts, experts, top, scale);
+}
+
+extern "C" int rl_router(const void* x, const float* w, float* route, int tokens, int k, int experts, int top,
+                         float scale, int act_type, hipStream_t stream) {
+    if (tokens <= 0) return RL_OK;
+    if (k < 1 || experts < 1 || experts > ROUTE_MAX_EXPERTS || top < 1 || top > experts) return RL_ERR_ARG;
+    dim3 grid((tokens + 3) / 4), block(256);
+    const size_t lds = (size_t)4 * experts * sizeof(float);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(router_kernel<float>, grid, block, lds, stream, (const float*)x, w, route, tokens, k,
+                           experts, top, scale);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(router_kernel<bf16_t>, grid, block, lds, stream, (const bf16_t*)x, w, route, tokens, k,
+                           experts, top, scale);
+    else
+        return RL_ERR_ARG;
     return rl_launch_status();
 }
 

@@ -297,6 +297,23 @@ def route(logits: torch.Tensor, top: int, scale: float) -> None:
     _ok(core().rl_route(_p(logits), tokens, experts, top, ctypes.c_float(scale), _stream()), "rl_route")
 
 
+def router(x: torch.Tensor, w: torch.Tensor, top: int, scale: float) -> torch.Tensor:
+    """The experts' weights ``[tokens, experts]`` (float32) of rows ``x`` under the float32 router
+    matrix ``w [experts, k]``: the product in float32, softmax over all experts, the ``top``
+    largest scores over their sum (+ 1e-20) times ``scale``, 0 elsewhere.  One kernel; a token's
+    result does not depend on the rest of the step."""
+    tokens, k = x.shape
+    experts = w.shape[0]
+    _need(x, "x")
+    _need(w, "router matrix", torch.float32, (experts, k))
+    if not 1 <= top <= experts <= ROUTE_MAX_EXPERTS:
+        raise KernelError(f"the router kernel chooses 1 to {experts} of at most {ROUTE_MAX_EXPERTS} experts, not {top}")
+    out = torch.empty((tokens, experts), dtype=torch.float32, device=x.device)
+    _ok(core().rl_router(_p(x), _p(w), _p(out), tokens, k, experts, top, ctypes.c_float(scale), _tag(x.dtype), _stream()),
+        "rl_router")
+    return out
+
+
 GLU_ALPHA = 1.702  # the sigmoid's slope in the clamped gated activation
 
 
@@ -1145,18 +1162,18 @@ def _static(ctx) -> dict:
     return ctx.extra if static is None else static
 
 
-def _f32_tiles(ctx, group: int) -> tuple[torch.Tensor, int]:
-    """Tiles of 16 (token, head of the group) rows, request by request: ``[tiles, 3]`` int32
-    (first token of the request in the step, its tokens, first row of the tile).  A function of
-    the requests' token counts alone."""
-    key = ("f32_tiles", group)
+def _f32_tiles(ctx, group: int, tile_rows: int = 16) -> tuple[torch.Tensor, int]:
+    """Tiles of ``tile_rows`` (token, head of the group) rows, request by request: ``[tiles, 3]``
+    int32 (first token of the request in the step, its tokens, first row of the tile).  A function
+    of the requests' token counts alone."""
+    key = ("f32_tiles", group) if tile_rows == 16 else ("row_tiles", group, tile_rows)
     store = _static(ctx)
     made = store.get(key)
     if made is None:
         tiles: list[int] = []
         at = 0
         for n in ctx.h_seq_lens:
-            for row0 in range(0, n * group, 16):
+            for row0 in range(0, n * group, tile_rows):
                 tiles += [at, n, row0]
             at += n
         made = (upload_ints(tiles, ctx.token_ids.device), len(tiles) // 3)
@@ -1248,12 +1265,21 @@ def attention_tile(
         )
     if nkv > 65535 or window < 0 or keep_first < 0:
         raise KernelError(f"{nkv} kv heads, window {window}, {keep_first} kept positions")
-    tiles, num_tiles = _f32_tiles(ctx, nq // nkv)
+    lib = attention_tile_lib(d, dv)
+    group = nq // nkv
+    # a bfloat16 step with portions: tiles of several blocks of 16 rows, so that the keys a
+    # workgroup reads serve more rows (float32 keeps one order of summation, whatever the step)
+    tile_rows = 16
+    if q.dtype == torch.bfloat16 and max(ctx.h_seq_lens) * group > 16:
+        tile_rows = lib.rl_attn_tile_wide_rows()
+    tiles, num_tiles = _f32_tiles(ctx, group, tile_rows)
+    # few tiles (a step of single tokens, mostly): more waves a tile, fewer steps a wave
+    wide = int(num_tiles * nkv <= chip().units)
     _ok(
-        attention_tile_lib(d, dv).rl_attn_tile(
+        lib.rl_attn_tile(
             _p(q), _p(k_cache), _p(v_cache), _p(out), _p(tiles), num_tiles, _p(ctx.positions),
             _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv, window,
-            int(keep_first), int(bool(sink)), ctypes.c_float(scale), _tag(q.dtype), _stream(),
+            int(keep_first), int(bool(sink)), ctypes.c_float(scale), wide, tile_rows, _tag(q.dtype), _stream(),
         ),
         "rl_attn_tile",
     )

@@ -190,8 +190,7 @@ class RoutedExperts(FeedForward):
         self.down.bind(params[self.name + ".down"])
 
     def forward(self, x, ctx):
-        weights = self.router(x, out_dtype=torch.float32)  # logits, float32 product
-        ops.route(weights, self.top, self.route_scale)
+        weights = ops.router(x, self.router.weight, self.top, self.route_scale)  # float32 throughout
         hidden = self.up(x)
         ops.unary_act(hidden, hidden, self.activation, weights, self.expert_size)
         return self.down.deferred(hidden, ctx)

@@ -299,6 +299,15 @@ def test_router_weights(experts, top, scale):
     ops.route(got, top, scale)
     torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-6)
     assert ((got.cpu() > 0).sum(dim=1) == top).all()
+    # product and weights in one kernel, from rows of either type; a token alone gives the same bits
+    for dtype in (torch.float32, torch.bfloat16):
+        hx = h.to(dtype)
+        chosen, weight = plain_route(hx.float(), router, top, scale)
+        want = torch.zeros(tokens, experts).scatter_(1, chosen, weight)
+        fused = ops.router(hx.to(DEV), router.to(DEV), top, scale)
+        torch.testing.assert_close(fused.cpu(), want, rtol=1e-4, atol=1e-5)
+        alone = ops.router(hx[5:6].contiguous().to(DEV), router.to(DEV), top, scale)
+        assert torch.equal(alone[0], fused[5])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
