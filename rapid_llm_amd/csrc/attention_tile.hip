@@ -91,6 +91,19 @@ __device__ inline void store_quad(bf16_t* p, f32x4 v) {
     *reinterpret_cast<s16x4*>(p) = o;
 }
 
+// exponentials: float32 keeps the library's; bfloat16 works in powers of two (the scores are
+// multiplied by scale * log2(e)) on the hardware's instruction
+template <typename T>
+__device__ inline float fexp(float x);
+template <>
+__device__ inline float fexp<float>(float x) {
+    return expf(x);
+}
+template <>
+__device__ inline float fexp<bf16_t>(float x) {
+    return __builtin_amdgcn_exp2f(x);
+}
+
 // the four lanes (r, g = 0..3) that share a row: the same bits in each of them
 __device__ inline float row_max(float v) {
     v = fmaxf(v, __shfl_xor(v, 16, RL_WAVE));
@@ -111,8 +124,10 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     T* __restrict__ out, const int* __restrict__ tile_info, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int nq, int nkv, int window, int keep_first, int sink, float scale) {
+    int page_size, int nq, int nkv, int window, int keep_first, int sink, float scale,
+    float* __restrict__ part, int nsplit) {
     typedef typename Quad<T>::type quad;
+    if constexpr (sizeof(T) == 2) scale *= 1.4426950408889634f;  // scores in units of log2
     const int tile = blockIdx.x;
     const int hk = blockIdx.y;
     const int G = nq / nkv;
@@ -141,6 +156,20 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
         kstart[r] = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
     }
     const int blocks = min(R, (rows - row0 + 15) / 16);  // blocks of the tile that hold rows
+    // keys [all_lo, all_hi) are seen by every row of a block (none where the block is not full):
+    // a tile of keys inside needs no masks
+    int all_lo[R], all_hi[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int rf = row0 + 16 * r, rl = rf + 15;
+        all_lo[r] = 1;
+        all_hi[r] = 0;
+        if (rl < rows) {
+            const int pl = start + rl / G;
+            all_hi[r] = start + rf / G + 1;
+            all_lo[r] = (window > 0 && pl - window + 1 > 0) ? pl - window + 1 : 0;
+        }
+    }
 
     // the keys any row of the tile sees: the kept first ones, and from the first row's first key
     // (rows ascend with the tokens), in whole tiles of 16, up to the last row's own position
@@ -227,21 +256,29 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
     auto finish_block = [&](int kb, int r, f32x4 s, const quad (&vcur)[VB]) {
         // ---- this lane's keys kb + 4g + i of its own row ------------------------------------
         float tmax = -INFINITY;
+        if (kb >= all_lo[r] && kb + 16 <= all_hi[r]) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int key = kb + 4 * g + i;
-            const bool seen = row_ok[r] && key < kend[r] && (key >= kstart[r] || key < keep);
-            s[i] = seen ? s[i] * scale : -INFINITY;
-            tmax = fmaxf(tmax, s[i]);
+            for (int i = 0; i < 4; ++i) {
+                s[i] *= scale;
+                tmax = fmaxf(tmax, s[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kb + 4 * g + i;
+                const bool seen = row_ok[r] && key < kend[r] && (key >= kstart[r] || key < keep);
+                s[i] = seen ? s[i] * scale : -INFINITY;
+                tmax = fmaxf(tmax, s[i]);
+            }
         }
         tmax = row_max(tmax);
         const float m_new = fmaxf(m[r], tmax);
         float alpha = 1.f;  // no visible key so far and none here: nothing changes
         f32x4 p = (f32x4){0.f, 0.f, 0.f, 0.f};
         if (m_new != -INFINITY) {
-            alpha = expf(m[r] - m_new);  // m = -inf before the row's first key: 0
+            alpha = fexp<T>(m[r] - m_new);  // m = -inf before the row's first key: 0
 #pragma unroll
-            for (int i = 0; i < 4; ++i) p[i] = expf(s[i] - m_new);  // masked: exactly 0
+            for (int i = 0; i < 4; ++i) p[i] = fexp<T>(s[i] - m_new);  // masked: exactly 0
         }
         l[r] = l[r] * alpha + row_sum((p[0] + p[1]) + (p[2] + p[3]));
         m[r] = m_new;
@@ -268,12 +305,15 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
         }
     };
 
-    // The wave's tiles, in ascending order: those of the kept keys with index % AW == wave,
-    // then those of [lo, hi) with index % AW == wave.
-    constexpr int STEP = 16 * AW;
-    const int kept_mine = 16 * wave;
+    // The wave's tiles, in ascending order: those of the kept keys with index % units == unit,
+    // then those of [lo, hi) with index % units == unit.  A launch may deal a tile's keys to
+    // several workgroups (blockIdx.z of nsplit): the units are then all their waves.
+    const int units = AW * nsplit;
+    const int unit = blockIdx.z * AW + wave;
+    const int STEP = 16 * units;
+    const int kept_mine = 16 * unit;
     const int kept_tiles = kept_mine < kept_end ? (kept_end - kept_mine + STEP - 1) / STEP : 0;
-    const int mine = lo + 16 * ((wave - lo / 16) & (AW - 1));  // first tile >= lo with index % AW == wave
+    const int mine = lo + 16 * (((unit - lo / 16) % units + units) % units);  // first tile >= lo with index % units == unit
     const int late_tiles = mine < hi ? (hi - mine + STEP - 1) / STEP : 0;
     const int total = kept_tiles + late_tiles;
     auto kb_of = [&](int i) -> int {
@@ -359,7 +399,7 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
             const float m_w = fold_ml[w][r][0][lane], l_w = fold_ml[w][r][1][lane];
             const float m_new = fmaxf(m[r], m_w);
             if (m_new == -INFINITY) continue;
-            const float fa = expf(m[r] - m_new), fb = expf(m_w - m_new);
+            const float fa = fexp<T>(m[r] - m_new), fb = fexp<T>(m_w - m_new);
             l[r] = l[r] * fa + l_w * fb;
 #pragma unroll
             for (int b = 0; b < VB; ++b)
@@ -369,8 +409,20 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
             m[r] = m_new;
         }
         if (!row_ok[r]) continue;
+        if (nsplit > 1) {
+            // this workgroup's share of the row's keys: sums, maximum and denominator go to the
+            // merge kernel as they are
+            float* prow = part + (((size_t)(at + tok[r]) * nq + head[r]) * nsplit + blockIdx.z) * (DV + 2);
+#pragma unroll
+            for (int b = 0; b < VB; ++b) *reinterpret_cast<f32x4*>(prow + 16 * b + 4 * g) = acc[r][b];
+            if (g == 0) {
+                prow[DV] = m[r];
+                prow[DV + 1] = l[r];
+            }
+            continue;
+        }
         // the key of score 0 that has no value: exp(0 - m) more in the denominator
-        if (sink) l[r] += expf(-m[r]);
+        if (sink) l[r] += fexp<T>(-m[r]);
         // acc[r][b][i] is channel 16b + 4g + i of the lane's row
         T* orow = out + ((size_t)(at + tok[r]) * nq + head[r]) * DV + 4 * g;
         const float inv = 1.f / l[r];
@@ -378,6 +430,29 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
         for (int b = 0; b < VB; ++b)
             store_quad(orow + 16 * b, (f32x4){acc[r][b][0] * inv, acc[r][b][1] * inv, acc[r][b][2] * inv,
                                               acc[r][b][3] * inv});
+    }
+}
+
+// Fold the shares of a row's keys that nsplit workgroups left (in order: the same bits every
+// run), add the sink's term and write the row.  One wave a row, a lane a channel (and more).
+__global__ __launch_bounds__(256) void attn_tile_merge_kernel(const float* __restrict__ part,
+                                                              bf16_t* __restrict__ out, int rows, int nsplit,
+                                                              int sink) {
+    const int row = blockIdx.x * 4 + threadIdx.x / RL_WAVE;
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    if (row >= rows) return;
+    const float* p = part + (size_t)row * nsplit * (DV + 2);
+    float top = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) top = fmaxf(top, p[s * (DV + 2) + DV]);
+    float den = 0.f;
+    for (int s = 0; s < nsplit; ++s)
+        den += __builtin_amdgcn_exp2f(p[s * (DV + 2) + DV] - top) * p[s * (DV + 2) + DV + 1];
+    if (sink) den += __builtin_amdgcn_exp2f(-top);
+    for (int c = lane; c < DV; c += RL_WAVE) {
+        float sum = 0.f;
+        for (int s = 0; s < nsplit; ++s)
+            sum += __builtin_amdgcn_exp2f(p[s * (DV + 2) + DV] - top) * p[s * (DV + 2) + c];
+        out[(size_t)row * DV + c] = float_to_bf16(sum / den);
     }
 }
 
@@ -398,7 +473,8 @@ extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_ca
                             const int* tile_info, int num_tiles, const int* positions,
                             const int* token_slot, const int* block_table, int table_stride,
                             int page_size, int nq, int nkv, int window, int keep_first, int sink,
-                            float scale, int wide, int tile_rows, int act_type, hipStream_t stream) {
+                            float scale, int nsplit, float* part, int tokens, int tile_rows, int act_type,
+                            hipStream_t stream) {
     if (num_tiles <= 0) return RL_OK;
     if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535 || window < 0 || keep_first < 0)
         return RL_ERR_ARG;
@@ -409,23 +485,30 @@ extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_ca
     (const TYPE*)q, (const TYPE*)k_cache, (const TYPE*)v_cache, (TYPE*)out, tile_info, positions, token_slot, \
         block_table, table_stride, page_size, nq, nkv, window, keep_first, sink, scale
     if (act_type == RL_BF16 && tile_rows == 16 * PB && PB > 1) {
-        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, PB>), grid, block, 0, stream, RL_TILE_ARGS(bf16_t));
+        if (nsplit != 1) return RL_ERR_ARG;
+        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, PB>), grid, block, 0, stream, RL_TILE_ARGS(bf16_t),
+                           nullptr, 1);
         return rl_launch_status();
     }
     if (tile_rows != 16) return RL_ERR_ARG;
-    // `wide` (bfloat16 only: the order of the sums changes with the number of waves): a launch of
-    // few tiles over many keys (single tokens) deals every tile's keys to as many waves as the
-    // fold's buffers allow, so that a wave walks a quarter of the steps
-    if (wide && act_type == RL_BF16) {
-        constexpr int WIDE = tileattn::DV <= 128 ? 16 : 8;
-        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, WIDE, 1>), grid, dim3(WIDE * RL_WAVE), 0, stream,
-                           RL_TILE_ARGS(bf16_t));
+    // nsplit > 1 (bfloat16 only: the order of the sums changes with it): a launch of few tiles
+    // over many keys (single tokens) deals every tile's keys to nsplit workgroups, whose shares
+    // the merge kernel folds; a compute unit's load path, not a wave's latency, bounds a tile
+    if (nsplit > 1) {
+        if (act_type != RL_BF16 || !part || nsplit > 64 || tokens < 1) return RL_ERR_ARG;
+        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, 1>), dim3(num_tiles, nkv, nsplit), block, 0, stream,
+                           RL_TILE_ARGS(bf16_t), part, nsplit);
+        const int rows = tokens * nq;
+        hipLaunchKernelGGL(tileattn::attn_tile_merge_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, part,
+                           (bf16_t*)out, rows, nsplit, sink);
         return rl_launch_status();
     }
     if (act_type == RL_F32)
-        hipLaunchKernelGGL((tileattn::attn_tile_kernel<float, AW, 1>), grid, block, 0, stream, RL_TILE_ARGS(float));
+        hipLaunchKernelGGL((tileattn::attn_tile_kernel<float, AW, 1>), grid, block, 0, stream, RL_TILE_ARGS(float),
+                           nullptr, 1);
     else if (act_type == RL_BF16)
-        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, 1>), grid, block, 0, stream, RL_TILE_ARGS(bf16_t));
+        hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, 1>), grid, block, 0, stream, RL_TILE_ARGS(bf16_t),
+                           nullptr, 1);
     else
         return RL_ERR_ARG;
 #undef RL_TILE_ARGS

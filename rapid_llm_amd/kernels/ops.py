@@ -1273,16 +1273,35 @@ def attention_tile(
     if q.dtype == torch.bfloat16 and max(ctx.h_seq_lens) * group > 16:
         tile_rows = lib.rl_attn_tile_wide_rows()
     tiles, num_tiles = _f32_tiles(ctx, group, tile_rows)
-    # few tiles (a step of single tokens, mostly): more waves a tile, fewer steps a wave
-    wide = int(num_tiles * nkv <= chip().units)
+    # few tiles over many keys (a step of single tokens, mostly): a tile's keys are dealt to
+    # several workgroups, on compute units of their own, and their shares merged
+    nsplit, part = 1, None
+    if q.dtype == torch.bfloat16 and tile_rows == 16:
+        nsplit = tile_splits(num_tiles * nkv, _static(ctx).get("context_bound", ctx.max_position + 1), window, keep_first)
+        if nsplit > 1:
+            part = torch.empty((tokens, nq, nsplit, dv + 2), dtype=torch.float32, device=q.device)
     _ok(
         lib.rl_attn_tile(
             _p(q), _p(k_cache), _p(v_cache), _p(out), _p(tiles), num_tiles, _p(ctx.positions),
             _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv, window,
-            int(keep_first), int(bool(sink)), ctypes.c_float(scale), wide, tile_rows, _tag(q.dtype), _stream(),
+            int(keep_first), int(bool(sink)), ctypes.c_float(scale), nsplit, _p(part), tokens, tile_rows,
+            _tag(q.dtype), _stream(),
         ),
         "rl_attn_tile",
     )
+
+
+_TILE_SPLIT_KEYS = 128  # fewest keys a workgroup's share of a tile is worth
+_TILE_MAX_SPLITS = 16
+
+
+def tile_splits(workgroups: int, span: int, window: int, keep_first: int, units: int | None = None) -> int:
+    """Workgroups a tile's keys are dealt to in a bfloat16 launch of ``workgroups`` (tile, kv head)
+    pairs over at most ``span`` keys: as many as give every compute unit one, each with a share
+    that is worth a workgroup."""
+    units = chip().units if units is None else units
+    keys = span if window <= 0 else min(span, window + keep_first + 16)
+    return max(1, min(_TILE_MAX_SPLITS, units // max(workgroups, 1), keys // _TILE_SPLIT_KEYS))
 
 
 def paged_attention(

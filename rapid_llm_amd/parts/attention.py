@@ -191,7 +191,9 @@ class GQAAttention(Mixer):
 
     def recorded_step_bytes(self, rows: int, context_bound: int, page_size: int) -> int:
         if self.extended:
-            return 0  # one kernel, nothing kept between two
+            # the shares of a tile's keys that several workgroups leave for the merge kernel
+            splits = ops.tile_splits(rows * self.nkv, context_bound, self.window, self.keep_first)
+            return 0 if splits == 1 else rows * self.nq * splits * (self.dv + 2) * 4
         return ops.decode_scratch_bytes(rows, self.nq, self.nkv, self.d, context_bound, page_size, self.window)
 
     # ---- step ------------------------------------------------------------------
