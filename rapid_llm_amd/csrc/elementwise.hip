@@ -744,6 +744,9 @@ __global__ __launch_bounds__(256) void router_kernel(const T* __restrict__ x, co
         for (int j = 0; j < 8; ++j) acc[j] = 0.f;
         const int ne = min(8, experts - e0);
         if (k % 4 == 0) {
+            // (unrolled: the loads of four iterations are asked for together; a step of a few
+            // tokens is all latency here)
+#pragma unroll 4
             for (int i = 4 * lane; i < k; i += 4 * RL_WAVE) {
                 const Vec4<T> xv = *reinterpret_cast<const Vec4<T>*>(xr + i);
                 float4 wv[8];
