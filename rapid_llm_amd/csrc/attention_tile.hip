@@ -80,8 +80,12 @@ __device__ inline f32x4 mma(s16x4 a, s16x4 b, f32x4 acc) {
 
 __device__ inline void to_quad(const f32x4& p, f32x4& out) { out = p; }
 __device__ inline void to_quad(const f32x4& p, s16x4& out) {
+    // the hardware's conversion (round to nearest even), two elements an instruction
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    bf16x4 b;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) out[i] = (short)float_to_bf16(p[i]).bits;
+    for (int i = 0; i < 4; ++i) b[i] = (__bf16)p[i];
+    out = __builtin_bit_cast(s16x4, b);
 }
 __device__ inline float quad_elem(const f32x4& q, int i) { return q[i]; }
 __device__ inline void store_quad(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
@@ -104,14 +108,22 @@ __device__ inline float fexp<bf16_t>(float x) {
     return __builtin_amdgcn_exp2f(x);
 }
 
-// the four lanes (r, g = 0..3) that share a row: the same bits in each of them
+// the four lanes (r, g = 0..3) that share a row: the same bits in each of them.  Two lane swaps
+// of gfx950 (the halves of the wave, then neighbouring rows of 16) instead of two trips through
+// the LDS crossbar; maximum and sum are commutative, so both partners of a swap get the same bits.
 __device__ inline float row_max(float v) {
-    v = fmaxf(v, __shfl_xor(v, 16, RL_WAVE));
-    return fmaxf(v, __shfl_xor(v, 32, RL_WAVE));
+    const unsigned u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned w = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+    const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ inline float row_sum(float v) {
-    v += __shfl_xor(v, 16, RL_WAVE);
-    return v + __shfl_xor(v, 32, RL_WAVE);
+    const unsigned u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned w = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 // tile_info: [tiles][3] = index of the request's first token in the step, its tokens in the

@@ -133,6 +133,7 @@ ATTENTION_CASES = [
     (3, 1, 12, 22, 4, 33, 9, True, [(0, 50), (41, 1), (42, 1), (100, 1)]),
     (6, 3, 24, 24, 4, 1, 2, True, [(0, 9), (5, 1)]),                      # a window of the own key alone
     (4, 1, 64, 32, 16, 1000, 30, True, [(3000, 1), (990, 40), (0, 1100)]),  # long contexts
+    (2, 1, 32, 16, 4, 0, 0, True, [(8300, 1), (8250, 60)]),  # more pages than a workgroup stages: the table is read
 ]
 
 
