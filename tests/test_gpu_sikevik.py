@@ -469,25 +469,29 @@ def test_trace_program(tmp_path):
 
 
 @pytest.mark.parametrize("use_graph", [False, True])
-@pytest.mark.parametrize("which", ["A", "C"])
-def test_greedy_generation_through_the_entry_point(tmp_path, which, use_graph):
+@pytest.mark.parametrize("which,dtype", [("A", "float32"), ("C", "float32"), ("C", "bfloat16")])
+def test_greedy_generation_through_the_entry_point(tmp_path, which, dtype, use_graph):
     """``LLM.generate``: scheduler, chunked prompts beside decoding requests, sampling kernels;
-    decode steps eagerly and replayed from graphs.  The plain implementation re-runs the whole
-    sequence for every token."""
+    decode steps eagerly and replayed from graphs (in bfloat16 a recorded step holds the shares
+    of a tile's keys and their merge).  The plain implementation re-runs the whole sequence for
+    every token; a bfloat16 engine may pick another of several nearly equal maxima."""
     from rapid_llm_amd import LLM, SamplingParams
 
     cfg, page, seed = SIKE[which]
     model_dir = make_model_dir(tmp_path, which)
     pcfg, pw = load_plain(model_dir)
     prompts = [random_tokens(n, cfg["vocab"], seed + n) for n in (1, 7, 30, 45)]
-    llm = LLM(str(model_dir), dtype="float32", page_size=page, num_pages=60, max_num_seqs=3, max_seq_len=96,
+    llm = LLM(str(model_dir), dtype=dtype, page_size=page, num_pages=60, max_num_seqs=3, max_seq_len=96,
               max_chunk_size=16, max_num_batched_tokens=32, use_cuda_graph=use_graph)
     outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_gen_len=24))
     for prompt, out in zip(prompts, outs):
         ids = list(prompt)
         for tok in out.token_ids:
             logits = plain_forward(pcfg, pw, ids)[-1]
-            assert float(logits.max() - logits[tok]) <= 1e-3, (len(prompt), len(ids))
+            if dtype == "float32":
+                assert float(logits.max() - logits[tok]) <= 1e-3, (len(prompt), len(ids))
+            else:
+                parity.assert_near_choice(logits, tok, f"generation/{which}/graph={use_graph}")
             ids.append(tok)
         assert len(out.token_ids) == 24
     llm.scheduler.cache.check_invariants()
