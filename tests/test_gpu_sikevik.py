@@ -240,7 +240,7 @@ def test_cache_write_of_value_heads_of_their_own_size(dtype, nq, nkv, d, dv, tok
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-@pytest.mark.parametrize("hidden", [96, 100, 256, 4100])
+@pytest.mark.parametrize("hidden", [96, 100, 256, 4100, 97, 18, 2050, 20000])
 def test_norm_behind_a_sublayer_add_and_next_norm_in_one_kernel(dtype, hidden):
     ops = _ops()
     tokens = 9
@@ -312,7 +312,7 @@ def test_router_weights(experts, top, scale):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-@pytest.mark.parametrize("hidden", [96, 100, 64])
+@pytest.mark.parametrize("hidden", [96, 100, 64, 99])
 def test_scaled_embedding_with_sinusoidal_positions(dtype, hidden):
     ops = _ops()
     table = torch.randn(50, hidden).to(dtype)
@@ -325,17 +325,18 @@ def test_scaled_embedding_with_sinusoidal_positions(dtype, hidden):
     want = table.float()[ids.long()] * 7.5 + plain_sinusoid(positions, hidden)
     torch.testing.assert_close(out.cpu(), want, rtol=1e-6, atol=1e-6)
     # position 0: sines 0, cosines 1
-    torch.testing.assert_close(out.cpu()[0] - table.float()[3] * 7.5, torch.tensor([0.0, 1.0]).repeat(hidden // 2),
-                               rtol=0, atol=1e-6)
+    torch.testing.assert_close(out.cpu()[0] - table.float()[3] * 7.5,
+                               torch.tensor([0.0, 1.0]).repeat((hidden + 1) // 2)[:hidden], rtol=0, atol=1e-6)
 
 
 def test_two_streams_side_by_side():
     ops = _ops()
-    a, b = torch.randn(7, 100), torch.randn(7, 100)
-    for dtype in (torch.float32, torch.bfloat16):
-        out = torch.empty((7, 200), dtype=dtype, device=DEV)
-        ops.pair_rows(a.to(DEV), b.to(DEV), out)
-        torch.testing.assert_close(out.cpu(), torch.cat([a, b], dim=1).to(dtype), rtol=0, atol=0)
+    for hidden in (100, 99):  # four channels a thread, and one
+        a, b = torch.randn(7, hidden), torch.randn(7, hidden)
+        for dtype in (torch.float32, torch.bfloat16):
+            out = torch.empty((7, 2 * hidden), dtype=dtype, device=DEV)
+            ops.pair_rows(a.to(DEV), b.to(DEV), out)
+            torch.testing.assert_close(out.cpu(), torch.cat([a, b], dim=1).to(dtype), rtol=0, atol=0)
 
 
 # --------------------------------------------------------------------------- #
